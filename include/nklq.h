@@ -1,0 +1,137 @@
+/*
+ * nklq.h — C-ABI of the MI355X (gfx950) 2-bit gradient quantizer.
+ *
+ * This is the boundary a binding of necklace's quantizer would load
+ * (dlopen / ctypes / cgo / JNI): plain pointers and sizes, no torch or numba
+ * types.  Every pointer marked "device" must be memory the current HIP device
+ * can address; `stream` is a hipStream_t passed as an opaque pointer (NULL =
+ * the device's default stream).  All entry points are asynchronous on
+ * `stream`, allocate nothing, keep no state between calls and may be called
+ * from several host threads at once.
+ *
+ * Bit layout (necklace/cuda/quantize.py:8-13, :34-51): codes are 2 bits,
+ * 01 = value >= t, 10 = value <= -t, 00 = in between, 16 codes per 32-bit
+ * word, the code of row 16*x + i of column y sits in bits [2i+1 : 2i] of
+ * word (x, y); bits of rows past the end are 0.  A flat vector of N elements
+ * is the matrix (N, 1): word w holds elements 16w .. 16w+15.
+ *
+ * Return value of the int entry points: 0 = success, < 0 = one of the
+ * NKLQ_E* argument errors below, > 0 = a hipError_t from the launch.
+ */
+#ifndef NKLQ_H
+#define NKLQ_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NKLQ_VERSION 100          /* 1.0.0 */
+#define NKLQ_CODES_PER_WORD 16    /* CMP_RATIO, necklace/cuda/quantize.py:8 */
+#define NKLQ_MAX_PAYLOADS_PER_LAUNCH 16
+
+#define NKLQ_OK 0
+#define NKLQ_ENULL (-1)   /* a required pointer is NULL */
+#define NKLQ_EALIGN (-2)  /* a pointer is not 4-byte aligned */
+#define NKLQ_ERANGE (-3)  /* a size or count is out of range */
+#define NKLQ_EALIAS (-4)  /* outputs overlap in a way the call cannot honour */
+
+/*
+ * Threshold-quantize an fp32 matrix to 2-bit codes and write the residual.
+ * Replaces the kernel cu_knl_matrix_quantize_e (necklace/cuda/quantize.py:16-51)
+ * and its launch wrapper cu_fn_matrix_quantize_e (:96-115).
+ *
+ *   g      device, fp32 [n_rows, n_cols] row-major: the matrix A of the reference
+ *   r_in   device, fp32 same shape: residual carried from the previous step;
+ *          read only when add_residual != 0 (may be NULL otherwise)
+ *   r_out  device, fp32 same shape: the matrix R of the reference (every
+ *          element is written).  May be the same pointer as r_in (in-place
+ *          error feedback) or as g; any other overlap is undefined.
+ *   c      device, uint32 [ceil(n_rows/16), n_cols] row-major: the matrix C
+ *          (every word is overwritten, whatever it held)
+ *   thrd   the threshold; it crosses as C float, i.e. rounded to fp32 exactly
+ *          like the jit signature '(..., float32)' at quantize.py:16 does
+ *   add_residual  0: a = g (the reference kernel as is)
+ *                 1: a = fl32(g + r_in) (error-feedback step), then as above
+ *
+ * Per element: a >= t -> code 01, r_out = fl32(a - t); else a <= -t -> code 10,
+ * r_out = fl32(a + t); else code 00, r_out = a (same bits).  NaN takes the
+ * last branch.  The column guard is y < n_cols (the reference tests y against
+ * n_rows, quantize.py:29-31, which is the same thing on the square inputs it
+ * is defined for).  n_rows == 0 or n_cols == 0 is a successful no-op.
+ */
+int nklq_quantize_f32(const float* g, const float* r_in, float* r_out, uint32_t* c,
+                      uint64_t n_rows, uint64_t n_cols, float thrd, int add_residual,
+                      void* stream);
+
+/*
+ * Unpack 2-bit codes to {+t, -t, 0.0f}, overwriting `out`.
+ * Replaces cu_knl_matrix_dequantize_e (necklace/cuda/quantize.py:56-87) and
+ * cu_fn_matrix_dequantize_e (:118-134).  Code 11 decodes to +0.0f (the
+ * reference's `else` branch, :86-87); bits of rows >= n_rows are never used.
+ * The reference's third argument R is unused by its kernel and has no
+ * counterpart here.
+ *
+ *   out  device, fp32 [n_rows, n_cols]     c  device, uint32 [ceil(n_rows/16), n_cols]
+ */
+int nklq_dequantize_f32(float* out, const uint32_t* c, uint64_t n_rows, uint64_t n_cols,
+                        float thrd, void* stream);
+
+/*
+ * Receive side: unpack k_payloads flat code vectors and sum them, in payload
+ * order, into one fp32 vector:
+ *     s = accumulate ? acc[j] : +0.0f;
+ *     for p = 0 .. k_payloads-1:  s = fl32(s + decode(payloads[p], j));
+ *     acc[j] = s;
+ * The order is part of the contract (fp32 sums of {0, +t, -t} depend on it).
+ * This is the "decompress and sum over workers" step that necklace's trainer
+ * hands to mxprms.grads_do_nccl(..., grad_comp_cfg=...) (call site
+ * necklace/trainer/tnopmx.py:334-337; that module is not in the reference
+ * tree), built on the decode of quantize.py:80-87.
+ *
+ *   acc       device, fp32 [n]
+ *   payloads  HOST array of k_payloads device pointers, each uint32 [ceil(n/16)];
+ *             read during the call only (the pointers travel as kernel
+ *             arguments; nothing is copied to or allocated on the device).
+ *             More than NKLQ_MAX_PAYLOADS_PER_LAUNCH payloads are processed
+ *             by consecutive launches that continue the same running sum.
+ *   k_payloads >= 1;  n == 0 is a successful no-op.
+ */
+int nklq_dequant_accumulate_f32(float* acc, const uint32_t* const* payloads, int k_payloads,
+                                uint64_t n, float thrd, int accumulate, void* stream);
+
+/*
+ * Number of uint32 words of the packed matrix: ceil(n_rows/16) * n_cols
+ * (the `m` of necklace/cuda/quantize.py:145-147 times the column count).
+ */
+uint64_t nklq_packed_words(uint64_t n_rows, uint64_t n_cols);
+
+/* Text for a return value of the entry points above (static storage). */
+const char* nklq_strerror(int code);
+
+/* NKLQ_VERSION the library was built from. */
+int nklq_version(void);
+
+/*
+ * Launch-geometry knobs, the counterpart of the reference wrapper's bpg/tpb
+ * keyword arguments (necklace/cuda/quantize.py:98,120).  Results never depend
+ * on them.  which: 0 = elements per lane in flight for the flat quantizer
+ * (4, 8 or 16), 1 = workgroups per compute unit for the streaming kernels
+ * (0 = one workgroup per tile, no grid-stride loop), 2 = non-temporal
+ * loads/stores (0/1).  Returns the previous value, or NKLQ_ERANGE.
+ * value < 0 only queries.
+ */
+int nklq_tune(int which, int value);
+
+/*
+ * Measurement aid, not part of the quantizer: dst[i] = src[i] for n fp32
+ * elements with the same 128-bit access pattern the quantizer uses.  Used to
+ * calibrate HBM counters and to quote a copy bandwidth beside the kernels.
+ */
+int nklq_copy_f32(float* dst, const float* src, uint64_t n, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NKLQ_H */
