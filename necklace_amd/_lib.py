@@ -1,0 +1,75 @@
+"""ctypes binding of libnklq.so (declarations: include/nklq.h).
+
+There is no fallback: if the library is missing or a call fails, an exception
+is raised.  Nothing here computes on the CPU.
+"""
+import ctypes as ct
+import os
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+SO_PATH = os.path.join(_PKG, "libnklq.so")
+
+NKLQ_MAX_PAYLOADS_PER_LAUNCH = 16
+
+SYMBOLS = (
+    "nklq_quantize_f32", "nklq_dequantize_f32", "nklq_dequant_accumulate_f32",
+    "nklq_packed_words", "nklq_strerror", "nklq_version", "nklq_tune", "nklq_copy_f32",
+)
+
+_lib = None
+
+
+class NklqError(RuntimeError):
+    def __init__(self, code, text):
+        super().__init__(f"libnklq error {code}: {text}")
+        self.code = code
+
+
+def lib():
+    """The loaded library; raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(SO_PATH):
+        raise ImportError(
+            f"{SO_PATH} is missing: build it with `python -m necklace_amd.csrc.build` "
+            "(needs hipcc; there is no CPU fallback)")
+    L = ct.CDLL(SO_PATH)
+    vp, u64, f32, i32 = ct.c_void_p, ct.c_uint64, ct.c_float, ct.c_int
+    L.nklq_quantize_f32.argtypes = [vp, vp, vp, vp, u64, u64, f32, i32, vp]
+    L.nklq_quantize_f32.restype = i32
+    L.nklq_dequantize_f32.argtypes = [vp, vp, u64, u64, f32, vp]
+    L.nklq_dequantize_f32.restype = i32
+    L.nklq_dequant_accumulate_f32.argtypes = [vp, ct.POINTER(vp), i32, u64, f32, i32, vp]
+    L.nklq_dequant_accumulate_f32.restype = i32
+    L.nklq_packed_words.argtypes = [u64, u64]
+    L.nklq_packed_words.restype = u64
+    L.nklq_strerror.argtypes = [i32]
+    L.nklq_strerror.restype = ct.c_char_p
+    L.nklq_version.argtypes = []
+    L.nklq_version.restype = i32
+    L.nklq_tune.argtypes = [i32, i32]
+    L.nklq_tune.restype = i32
+    L.nklq_copy_f32.argtypes = [vp, vp, u64, vp]
+    L.nklq_copy_f32.restype = i32
+    _lib = L
+    return L
+
+
+def check(code):
+    if code != 0:
+        raise NklqError(code, lib().nklq_strerror(code).decode())
+
+
+def packed_words(n_rows, n_cols=1):
+    return int(lib().nklq_packed_words(n_rows, n_cols))
+
+
+TUNE_ELEMS_PER_LANE, TUNE_WG_PER_CU, TUNE_NONTEMPORAL = 0, 1, 2
+
+
+def tune(which, value=-1):
+    r = lib().nklq_tune(which, value)
+    if r < 0:
+        raise ValueError(f"nklq_tune({which}, {value}) rejected")
+    return r

@@ -1,0 +1,50 @@
+"""Device helpers with the names of necklace/cuda/nbutils.py:11-39, on PyTorch-ROCm.
+
+numba is gone: a "device array" is a torch tensor on the GPU, a "stream" is a
+torch.cuda.Stream (a HIP stream).
+"""
+import ctypes as ctp
+
+import numpy as np
+import torch
+
+
+def cuda_select_device(dev_i):
+    """necklace/cuda/nbutils.py:11-17."""
+    torch.cuda.set_device(int(dev_i))
+
+
+def cuda_current_context():
+    """necklace/cuda/nbutils.py:20-22; HIP has no user-visible context object, the device is it."""
+    return torch.device("cuda", torch.cuda.current_device())
+
+
+def cuda_stream():
+    """necklace/cuda/nbutils.py:25-27: a new stream (default priority)."""
+    return torch.cuda.Stream()
+
+
+def cuda_to_device(A, stream=None):
+    """necklace/cuda/nbutils.py:30-34: copy a host array to the current GPU."""
+    if isinstance(A, torch.Tensor):
+        t = A
+    else:
+        t = torch.from_numpy(np.ascontiguousarray(A))
+    if stream is None:
+        return t.to("cuda")
+    with torch.cuda.stream(stream):
+        return t.to("cuda", non_blocking=False)
+
+
+def cuda_devarr_c_void_p(d_arr):
+    """necklace/cuda/nbutils.py:37-39: device address as ctypes.c_void_p."""
+    return ctp.c_void_p(d_arr.data_ptr())
+
+
+def stream_handle(stream=None, device=None):
+    """hipStream_t (as int) of `stream`; None means torch's current stream on `device`."""
+    if stream is None:
+        return torch.cuda.current_stream(device).cuda_stream
+    if isinstance(stream, int):
+        return stream
+    return stream.cuda_stream

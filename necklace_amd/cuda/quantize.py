@@ -1,0 +1,214 @@
+"""2-bit gradient quantization on MI355X — drop-in for necklace/cuda/quantize.py.
+
+Same public names and keyword arguments as the reference module; the work is
+done by the HIP kernels of libnklq.so (include/nklq.h).  Differences a caller
+can see, all deliberate:
+
+* `A`, `C`, `R` are torch tensors on the GPU (or numpy arrays with
+  ``to_device=True``) instead of numba device arrays; `C` may be torch.uint32
+  or torch.int32 (same bits);
+* 1-D tensors are accepted and mean the matrix (N, 1): word w packs elements
+  16w .. 16w+15;
+* `bpg` / `tpb` are accepted and ignored: the library sizes its own launch and
+  always covers the whole input, where the reference's fixed (bpg, bpg) grid
+  covers at most 16*bpg*tpb/16 word rows x bpg*tpb columns
+  (necklace/cuda/quantize.py:98,112);
+* the column guard is ``y < A.shape[1]``; the reference tests y against
+  ``A.shape[0]`` (:29-31), which only works for square inputs;
+* extra keyword arguments: ``add_residual`` (error feedback: a = A + R before
+  quantizing, R updated in place) and ``sync`` (the reference always blocks
+  until the stream is idle, :104; pass ``sync=False`` to stay asynchronous).
+"""
+import ctypes as ct
+
+import numpy as np
+import torch
+
+from .. import _lib
+from . import nbutils
+
+CMP_RATIO = 16  # necklace/cuda/quantize.py:8
+
+g = 0b01  # a >= thrd
+e = 0b00  # -thrd < a < thrd
+l = 0b10  # a <= -thrd
+msk = 0b11  # or mask
+
+_WORD_DTYPES = (torch.int32, torch.uint32)
+
+
+def packed_rows(n):
+    """m of necklace/cuda/quantize.py:145-147."""
+    return (n + CMP_RATIO - 1) // CMP_RATIO
+
+
+def _shape2(t):
+    if t.dim() == 1:
+        return t.shape[0], 1
+    return t.shape[0], t.shape[1]
+
+
+def _check_f32(name, t):
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name}: expected a torch tensor, got {type(t).__name__}")
+    if t.dtype != torch.float32:
+        raise TypeError(f"{name}: expected float32, got {t.dtype}")
+    if t.dim() not in (1, 2):
+        raise TypeError(f"{name}: expected 1 or 2 dimensions, got {t.dim()}")
+    if not t.is_cuda:
+        raise TypeError(f"{name}: expected a GPU tensor (pass to_device=True for host arrays)")
+    if not t.is_contiguous():
+        raise ValueError(f"{name}: must be contiguous")
+
+
+def _check_words(name, t, n, k, ndim):
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name}: expected a torch tensor, got {type(t).__name__}")
+    if t.dtype not in _WORD_DTYPES:
+        raise TypeError(f"{name}: expected uint32 or int32, got {t.dtype}")
+    if not t.is_cuda:
+        raise TypeError(f"{name}: expected a GPU tensor")
+    if not t.is_contiguous():
+        raise ValueError(f"{name}: must be contiguous")
+    want = (packed_rows(n),) if ndim == 1 else (packed_rows(n), k)
+    if tuple(t.shape) != want and not (ndim == 1 and tuple(t.shape) == (want[0], 1)):
+        raise ValueError(f"{name}: shape {tuple(t.shape)} does not match {want} for {n} rows")
+
+
+def _to_device(x):
+    if isinstance(x, torch.Tensor):
+        return x.cuda()
+    return torch.from_numpy(np.ascontiguousarray(x)).cuda()
+
+
+def _finish(stream, device, sync):
+    if not sync:
+        return
+    if stream is None:
+        torch.cuda.current_stream(device).synchronize()
+    elif isinstance(stream, int):
+        torch.cuda.synchronize(device)
+    else:
+        stream.synchronize()
+
+
+def _quantize(A, C, R, thrd, add_residual, stream, sync):
+    _check_f32("A", A)
+    _check_f32("R", R)
+    if A.shape != R.shape:
+        raise ValueError(f"A {tuple(A.shape)} and R {tuple(R.shape)} differ in shape")
+    n, k = _shape2(A)
+    _check_words("C", C, n, k, A.dim())
+    if not (A.device == R.device == C.device):
+        raise ValueError("A, C and R must be on the same GPU")
+    with torch.cuda.device(A.device):
+        h = nbutils.stream_handle(stream, A.device)
+        _lib.check(_lib.lib().nklq_quantize_f32(
+            A.data_ptr(), R.data_ptr() if add_residual else None, R.data_ptr(), C.data_ptr(),
+            n, k, float(thrd), 1 if add_residual else 0, h))
+        _finish(stream, A.device, sync)
+
+
+def _dequantize(A, C, thrd, stream, sync):
+    _check_f32("A", A)
+    n, k = _shape2(A)
+    _check_words("C", C, n, k, A.dim())
+    if A.device != C.device:
+        raise ValueError("A and C must be on the same GPU")
+    with torch.cuda.device(A.device):
+        h = nbutils.stream_handle(stream, A.device)
+        _lib.check(_lib.lib().nklq_dequantize_f32(A.data_ptr(), C.data_ptr(), n, k, float(thrd), h))
+        _finish(stream, A.device, sync)
+
+
+class _Kernel:
+    """Stands in for a numba kernel object: ``knl[grid, block, stream](A, C, R, thrd)``.
+
+    (necklace/cuda/quantize.py:112,134.)  Grid and block are accepted and
+    ignored; the launch is asynchronous on `stream`, as a numba launch is.
+    """
+
+    def __init__(self, name, fn):
+        self.__name__ = name
+        self._fn = fn
+
+    def __getitem__(self, cfg):
+        if not isinstance(cfg, tuple):
+            cfg = (cfg,)
+        stream = cfg[2] if len(cfg) > 2 else None
+        return lambda A, C, R, thrd=0.3: self._fn(A, C, R, thrd, stream)
+
+    def __call__(self, A, C, R, thrd=0.3):
+        return self._fn(A, C, R, thrd, None)
+
+
+cu_knl_matrix_quantize_e = _Kernel(
+    "cu_knl_matrix_quantize_e",
+    lambda A, C, R, thrd, stream: _quantize(A, C, R, thrd, False, stream or None, False))
+cu_knl_matrix_dequantize_e = _Kernel(
+    "cu_knl_matrix_dequantize_e",
+    lambda A, C, R, thrd, stream: _dequantize(A, C, thrd, stream or None, False))
+
+
+def cu_fn_matrix_quantize_e(A, C, R, thrd=0.3,
+                            bpg=4, tpb=128,
+                            to_device=False, stream=None,
+                            add_residual=False, sync=True):
+    """Quantize A to 2-bit codes in C and write the residual to R.
+
+    Signature of necklace/cuda/quantize.py:96-99.  With ``to_device=True`` the
+    inputs are host arrays, copied to the GPU first; the results stay on the GPU
+    (the reference does the same and drops them, :105-115) and are returned as
+    ``(dA, dC, dR)``.
+    """
+    if to_device:
+        A, R, C = _to_device(A), _to_device(R), _to_device(C)
+    _quantize(A, C, R, thrd, add_residual, stream or None, sync)
+    return (A, C, R) if to_device else None
+
+
+def cu_fn_matrix_dequantize_e(A, C, R, thrd=0.3,
+                              bpg=4, tpb=128,
+                              to_device=False, stream=None, sync=True):
+    """Decode C into A (overwrite).  Signature of necklace/cuda/quantize.py:118-121.
+
+    R is unused, exactly as in the reference kernel (:56-87); None is accepted.
+    """
+    if to_device:
+        A, C = _to_device(A), _to_device(C)
+        R = _to_device(R) if R is not None else None
+    _dequantize(A, C, thrd, stream or None, sync)
+    return (A, C, R) if to_device else None
+
+
+# ------------------------------------------------------------------ receive side
+
+def cu_fn_dequantize_accumulate_e(acc, payloads, thrd=0.3, accumulate=False, stream=None, sync=True):
+    """acc[j] = (((s0 + d_0[j]) + d_1[j]) + ...), d_p = decode of payloads[p], in list order.
+
+    s0 is +0.0 (``accumulate=False``) or the value already in `acc`.  `acc` is a
+    1-D float32 GPU tensor of n elements; `payloads` a sequence of 1-D word
+    tensors of ceil(n/16) words each, or one 2-D tensor [K, ceil(n/16)].  This is
+    the decompress-and-sum step the compressed gradient exchange needs
+    (necklace/trainer/tnopmx.py:334-337); the decode is quantize.py:80-87.
+    """
+    _check_f32("acc", acc)
+    if acc.dim() != 1:
+        raise TypeError("acc: expected 1 dimension")
+    n = acc.shape[0]
+    if isinstance(payloads, torch.Tensor):
+        if payloads.dim() != 2:
+            raise TypeError("payloads: expected a sequence of 1-D tensors or one 2-D tensor")
+        payloads = list(payloads.unbind(0))
+    if len(payloads) < 1:
+        raise ValueError("payloads: at least one is required")
+    for i, p in enumerate(payloads):
+        _check_words(f"payloads[{i}]", p, n, 1, 1)
+        if p.device != acc.device:
+            raise ValueError("acc and payloads must be on the same GPU")
+    ptrs = (ct.c_void_p * len(payloads))(*[p.data_ptr() for p in payloads])
+    with torch.cuda.device(acc.device):
+        h = nbutils.stream_handle(stream, acc.device)
+        _lib.check(_lib.lib().nklq_dequant_accumulate_f32(
+            acc.data_ptr(), ptrs, len(payloads), n, float(thrd), 1 if accumulate else 0, h))
+        _finish(stream, acc.device, sync)

@@ -1,0 +1,196 @@
+"""HIP kernels vs the CPU oracle, through the C-ABI, bit for bit.
+
+Codes and residuals: exact bits (NaN matches NaN).  Sums: 0 ULP.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from conftest import assert_bits_equal, assert_words_equal, bits_to_f32, kat_quant_cases
+from gpu_util import dev, gpu_dequantize, gpu_quantize, host_words, pack_codes_np, words_like
+from necklace_amd import _lib
+from necklace_amd.cuda import quantize as q
+
+pytestmark = pytest.mark.gpu
+
+FLAT_SIZES = list(range(1, 50)) + [63, 64, 65, 255, 256, 257, 1023, 1024, 1025, 4095, 4096, 4097,
+                                   8191, 12289, 65536 + 5, 1048576 + 17]
+
+
+def _knobs():
+    """Launch geometries to run every flat test under; results must not depend on them."""
+    return [(16, 0, 1), (8, 0, 0), (4, 2, 1), (16, 1, 0), (16, 8, 1)]
+
+
+@pytest.fixture(params=_knobs(), ids=lambda k: f"epl{k[0]}-wg{k[1]}-nt{k[2]}")
+def knobs(request):
+    old = [_lib.tune(i) for i in range(3)]
+    for i, v in enumerate(request.param):
+        _lib.tune(i, v)
+    yield request.param
+    for i, v in enumerate(old):
+        _lib.tune(i, v)
+
+
+def test_kat_vectors_on_gpu(kat):
+    for name, a, t, words, r, _ in kat_quant_cases(kat):
+        C, R = gpu_quantize(a, t)
+        assert_words_equal(C, words, name)
+        assert_bits_equal(R, r, name)
+    for v in kat["dequantize"]:
+        t = float(bits_to_f32([v["thrd_bits"]])[0])
+        words = np.array([int(h, 16) for h in v["words"]], dtype=np.uint32)
+        assert_bits_equal(gpu_dequantize(words, v["n"], t), bits_to_f32(v["out_bits"]), v["name"])
+    for v in kat["accumulate"]:
+        t = float(bits_to_f32([v["thrd_bits"]])[0])
+        pl = [dev(np.array([int(h, 16) for h in p], dtype=np.uint32)) for p in v["payload_words"]]
+        acc = torch.full((v["n"],), 3.0, device="cuda")
+        q.cu_fn_dequantize_accumulate_e(acc, pl, t)
+        assert_bits_equal(acc.cpu().numpy(), bits_to_f32(v["acc_bits"]), v["name"])
+
+
+def test_flat_sizes_all_knobs(knobs):
+    for n in FLAT_SIZES:
+        rng = np.random.default_rng(n)
+        a = rng.normal(0, 0.01, n).astype(np.float32)
+        r0 = rng.normal(0, 0.004, n).astype(np.float32)
+        Cw, Rw = oracle.c.quantize(a, 0.005)
+        C, R = gpu_quantize(a, 0.005)
+        assert_words_equal(C, Cw, f"plain n={n}")
+        assert_bits_equal(R, Rw, f"plain n={n}")
+        Cw, Rw = oracle.c.quantize(a, 0.005, R_in=r0)
+        C, R = gpu_quantize(a, 0.005, r_in_np=r0)
+        assert_words_equal(C, Cw, f"fused n={n}")
+        assert_bits_equal(R, Rw, f"fused n={n}")
+        assert_bits_equal(gpu_dequantize(Cw, n, 0.005), oracle.c.dequantize(Cw, n, 0.005), f"deq n={n}")
+
+
+@pytest.mark.parametrize("og,orr", [(1, 1), (2, 3), (3, 0), (0, 1), (1, 2)])
+def test_flat_views_at_any_element_offset(og, orr, knobs):
+    """Gradient views cut out of a flat buffer: base addresses only 4-byte aligned."""
+    for n in (5, 100, 4096 + 3, 70001):
+        rng = np.random.default_rng(n + og * 10 + orr)
+        a = rng.normal(0, 1e-3, n).astype(np.float32)
+        r0 = rng.normal(0, 5e-4, n).astype(np.float32)
+        Cw, Rw = oracle.c.quantize(a, 1e-3, R_in=r0)
+        C, R = gpu_quantize(a, 1e-3, r_in_np=r0, offset=(og, orr))
+        assert_words_equal(C, Cw, f"n={n}")
+        assert_bits_equal(R, Rw, f"n={n}")
+        assert_bits_equal(gpu_dequantize(Cw, n, 1e-3, offset=orr), oracle.c.dequantize(Cw, n, 1e-3))
+
+
+@pytest.mark.parametrize("thrd", [0.005, 1e-3, 2e-3, 1e-2, 0.3, 0.5, 0.0, -0.25, 1e-45])
+def test_every_float_near_the_threshold_and_specials(thrd):
+    t = np.float32(thrd if thrd > 0 else 0.25)
+    tb = int(t.view(np.uint32))
+    pos = np.arange(tb - 64, tb + 65, dtype=np.int64).astype(np.uint32)
+    special = np.array([0x00000000, 0x80000000, 0x00000001, 0x80000001, 0x007FFFFF, 0x807FFFFF,
+                        0x00800000, 0x80800000, 0x7F7FFFFF, 0xFF7FFFFF, 0x7F800000, 0xFF800000,
+                        0x7FC00000, 0xFFC00001, 0x7F800001], dtype=np.uint32)
+    a = np.concatenate([pos, pos | np.uint32(0x80000000), special]).view(np.float32)
+    # plain: denormals, signed zeros, infinities and NaN go through untouched or shifted by t
+    Cw, Rw = oracle.c.quantize(a, thrd)
+    C, R = gpu_quantize(a, thrd)
+    assert_words_equal(C, Cw)
+    assert_bits_equal(R, Rw)
+    # fused with residuals that land the sum on and around the threshold
+    r0 = (np.float32(t) - a).astype(np.float32)
+    r0[~np.isfinite(r0)] = 0
+    Cw, Rw = oracle.c.quantize(a, thrd, R_in=r0)
+    C, R = gpu_quantize(a, thrd, r_in_np=r0)
+    assert_words_equal(C, Cw)
+    assert_bits_equal(R, Rw)
+
+
+@pytest.mark.parametrize("n,k", [(224, 224), (17, 3), (33, 7), (16, 4), (100, 64), (5, 256), (1000, 12),
+                                 (1, 1), (31, 2), (64, 1000), (513, 260)])
+def test_matrix_layout(n, k):
+    """Column-packed (n, k) form; (224, 224) with values in [-1, 0) and thrd 0.5 is the
+    reference's own smoke input (necklace/cuda/quantize.py:141-153)."""
+    rng = np.random.default_rng(n * 7 + k)
+    A = (rng.random((n, k)).astype(np.float32) - np.float32(1.0))
+    R0 = rng.normal(0, 0.3, (n, k)).astype(np.float32)
+    Cw, Rw = oracle.c.quantize(A, 0.5)
+    C, R = gpu_quantize(A, 0.5)
+    assert_words_equal(C, Cw)
+    assert_bits_equal(R, Rw)
+    Cw2, Rw2 = oracle.c.quantize(A, 0.5, R_in=R0)
+    C, R = gpu_quantize(A, 0.5, r_in_np=R0)
+    assert_words_equal(C, Cw2)
+    assert_bits_equal(R, Rw2)
+    assert_bits_equal(gpu_dequantize(Cw, n, 0.5, k=k), oracle.c.dequantize(Cw, n, 0.5))
+    # all four codes, whatever sits in the words
+    junk = rng.integers(0, 2 ** 32, size=Cw.shape, dtype=np.uint64).astype(np.uint32)
+    assert_bits_equal(gpu_dequantize(junk, n, 0.5, k=k), oracle.c.dequantize(junk, n, 0.5))
+
+
+def test_in_place_forms():
+    """R may be A itself (plain), and the fused step updates R in place."""
+    rng = np.random.default_rng(99)
+    n = 10000 + 9
+    a = rng.normal(0, 0.01, n).astype(np.float32)
+    Cw, Rw = oracle.c.quantize(a, 0.005)
+    A = dev(a)
+    C = words_like(n)
+    q.cu_fn_matrix_quantize_e(A, C, A, 0.005)  # residual written over the input
+    assert_words_equal(host_words(C), Cw)
+    assert_bits_equal(A.cpu().numpy(), Rw)
+
+
+def test_reference_style_calls():
+    """kernel[grid, block, stream](...), to_device=True, explicit stream, uint32 words."""
+    rng = np.random.default_rng(5)
+    n = 224
+    A = (rng.random((n, n)).astype(np.float32) - np.float32(1.0))
+    Cw, Rw = oracle.c.quantize(A, 0.5)
+    # to_device=True with host arrays (necklace/cuda/quantize.py:105-108)
+    dA, dC, dR = q.cu_fn_matrix_quantize_e(A, np.zeros((14, n), np.uint32), np.empty_like(A), 0.5,
+                                           to_device=True)
+    assert dC.dtype == torch.uint32
+    assert_words_equal(host_words(dC), Cw)
+    assert_bits_equal(dR.cpu().numpy(), Rw)
+    # subscripted kernel object on a stream of its own (:112)
+    s = torch.cuda.Stream()
+    dA, dC2, dR2 = dev(A), words_like(n, n), torch.empty(n, n, device="cuda")
+    s.wait_stream(torch.cuda.current_stream())
+    q.cu_knl_matrix_quantize_e[(8, 8), (8, 128), s](dA, dC2, dR2, 0.5)
+    s.synchronize()
+    assert_words_equal(host_words(dC2), Cw)
+    dB = torch.empty(n, n, device="cuda")
+    q.cu_fn_matrix_dequantize_e(dB, dC2, dR2, 0.5, stream=s)
+    assert_bits_equal(dB.cpu().numpy(), oracle.c.dequantize(Cw, n, 0.5))
+
+
+@pytest.mark.parametrize("k_payloads", [1, 2, 8, 16, 17, 35])
+def test_accumulate_fixed_order(k_payloads, knobs):
+    for n in (1, 15, 16, 17, 1000 + 13, 4096, 100003):
+        rng = np.random.default_rng(n + k_payloads)
+        pl = []
+        for p in range(k_payloads):
+            codes = rng.choice([0, 1, 2, 3], size=n, p=[0.6, 0.19, 0.19, 0.02]).astype(np.uint32)
+            w = pack_codes_np(codes, n)
+            if n % 16:
+                w[-1] |= np.uint32((0xFFFFFFFF << (2 * (n % 16))) & 0xFFFFFFFF)  # garbage past the end
+            pl.append(w)
+        want = oracle.c.dequant_accumulate(pl, n, 1e-3)
+        acc = torch.full((n,), 5.0, device="cuda")
+        dpl = [dev(w) for w in pl]
+        q.cu_fn_dequantize_accumulate_e(acc, dpl, 1e-3)
+        assert_bits_equal(acc.cpu().numpy(), want, f"n={n}")
+        base = rng.normal(0, 1e-2, n).astype(np.float32)
+        want2 = oracle.c.dequant_accumulate(pl, n, 1e-3, acc=base)
+        acc2 = dev(base)
+        q.cu_fn_dequantize_accumulate_e(acc2, torch.stack(dpl), 1e-3, accumulate=True)
+        assert_bits_equal(acc2.cpu().numpy(), want2, f"n={n} accumulate")
+
+
+def test_round_trip_and_zero_residual_on_gpu():
+    rng = np.random.default_rng(21)
+    n = 1 << 20
+    a = rng.standard_t(3, n).astype(np.float32) * np.float32(1e-3)
+    C, R = gpu_quantize(a, 2e-3)
+    d = gpu_dequantize(C, n, 2e-3)
+    C2, R2 = gpu_quantize(d, 2e-3)
+    assert_words_equal(C2, C)
+    assert not R2.any()
