@@ -6,6 +6,12 @@ is raised.  Nothing here computes on the CPU.
 import ctypes as ct
 import os
 
+# torch first: it carries its own copy of the HIP runtime (soname libamdhip64.so.7).  Loaded
+# before libnklq.so, that copy also satisfies libnklq's dependency, so tensors and kernels
+# share one runtime; the other way round the process ends up with two runtimes and the second
+# one finds no device.
+import torch  # noqa: F401
+
 _PKG = os.path.dirname(os.path.abspath(__file__))
 SO_PATH = os.path.join(_PKG, "libnklq.so")
 

@@ -1,0 +1,170 @@
+"""The five benchmark workloads at their full sizes, HIP path vs the CPU oracle.
+
+Every comparison is on identical inputs: data is generated once (numpy on the
+host, or torch on the GPU and downloaded) and handed to both sides.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from conftest import assert_bits_equal, assert_words_equal
+from gpu_util import (dev, host_words, random_payloads_gpu, resnet50_segment_sizes, student_t3_gpu,
+                      words_like)
+from necklace_amd import _lib
+from necklace_amd.cuda import quantize as q
+
+pytestmark = pytest.mark.gpu
+
+
+def test_config1_flat_and_square():
+    """N = 1,048,576, g ~ N(0, 0.01), r = 0, thrd 0.005, one step; as the flat vector and as the
+    1024 x 1024 matrix the reference wrapper itself could run (bpg=8, tpb=128)."""
+    n = 1 << 20
+    rng = np.random.default_rng(20240101)
+    g = rng.normal(0, 0.01, n).astype(np.float32)
+    # flat, fused with a zero residual
+    want_c, want_r = oracle.c.quantize(g, 0.005, R_in=np.zeros(n, np.float32))
+    dg, dr, dc = dev(g), torch.zeros(n, device="cuda"), words_like(n)
+    q.cu_fn_matrix_quantize_e(dg, dc, dr, 0.005, add_residual=True)
+    assert_words_equal(host_words(dc), want_c)
+    assert_bits_equal(dr.cpu().numpy(), want_r)
+    assert host_words(dc).size == 65536
+    # square, the reference kernel as is
+    G = g.reshape(1024, 1024)
+    want_c2, want_r2 = oracle.c.quantize(G, 0.005)
+    dG, dR, dC = dev(G), torch.empty(1024, 1024, device="cuda"), words_like(1024, 1024)
+    q.cu_fn_matrix_quantize_e(dG, dC, dR, 0.005, bpg=8, tpb=128)
+    assert_words_equal(host_words(dC), want_c2)
+    assert_bits_equal(dR.cpu().numpy(), want_r2)
+    assert want_c2.shape == (64, 1024)
+    # same numbers, different bit layout: the two packings must not be confused
+    assert not np.array_equal(want_c2.reshape(-1), want_c)
+    dB = torch.empty(1024, 1024, device="cuda")
+    q.cu_fn_matrix_dequantize_e(dB, dC, dR, 0.005)
+    assert_bits_equal(dB.cpu().numpy(), oracle.c.dequantize(want_c2, 1024, 0.005))
+
+
+def test_config2_resnet50_ten_error_feedback_steps():
+    """25,557,032 elements in 161 segments (sigma log-uniform in [1e-4, 1e-2]), thrd 1e-3, 10 steps,
+    residual carried; codes and residual compared after every step."""
+    sizes = resnet50_segment_sizes()
+    n = sum(sizes)
+    rng = np.random.default_rng(2)
+    sigma = np.repeat((10.0 ** rng.uniform(-4, -2, len(sizes))).astype(np.float32), sizes)
+    r_host = np.zeros(n, dtype=np.float32)
+    c_host = np.zeros((n + 15) // 16, dtype=np.uint32)
+    dr, dc = torch.zeros(n, device="cuda"), words_like(n)
+    assert n % 16 == 8
+    sent = 0
+    for step in range(10):
+        g = np.random.default_rng([2, step]).standard_normal(n, dtype=np.float32) * sigma
+        oracle.c.fused_quantize_inplace(g, r_host, c_host, 1e-3)
+        q.cu_fn_matrix_quantize_e(dev(g), dc, dr, 1e-3, add_residual=True)
+        got_c = host_words(dc)
+        assert_words_equal(got_c, c_host, f"step {step}")
+        assert_bits_equal(dr.cpu().numpy(), r_host, f"step {step}")
+        assert int(got_c[-1]) >> 16 == 0  # the last word holds 8 codes
+        sent += int(np.count_nonzero(got_c))
+    assert sent > 0
+
+
+def test_config3_receive_side_64_buckets():
+    """64 buckets, lengths uniform in [1M, 8M] and not multiples of 16; per bucket the local payload
+    (quantize of a seeded gradient) and 7 peers (P(0)=0.9) are decoded and summed in order 0..7."""
+    rng = np.random.default_rng(3)
+    lens = []
+    while len(lens) < 64:
+        v = int(rng.integers(1_000_000, 8_000_001))
+        if v % 16:
+            lens.append(v)
+    thrd = 1e-3
+    total = 0
+    for b, n in enumerate(lens):
+        g = student_t3_gpu(n, 1000 + b, scale=1e-3)
+        local = words_like(n)
+        resid = torch.empty(n, device="cuda")
+        q.cu_fn_matrix_quantize_e(g, local, resid, thrd, sync=False)
+        peers = random_payloads_gpu(7, n, 2000 + b, garbage_tail=(b % 8 == 5))
+        acc = torch.full((n,), float("nan"), device="cuda")
+        payloads = [local] + list(peers.unbind(0))
+        q.cu_fn_dequantize_accumulate_e(acc, payloads, thrd)
+        host_pl = [host_words(p) for p in payloads]
+        want = oracle.c.dequant_accumulate(host_pl, n, thrd)
+        assert_bits_equal(acc.cpu().numpy(), want, f"bucket {b} n={n}")
+        total += n
+    assert 64_000_000 <= total <= 512_000_000
+
+
+def test_config4_gpt2_medium_fused_step_and_round_trip():
+    """354,823,168 elements, g = 1e-3 * Student-t(3), r0 ~ N(0, 1e-4), thrd 2e-3: one fused step
+    compared in full with the oracle, then the decode round trip."""
+    n, thrd = 354_823_168, 2e-3
+    g = student_t3_gpu(n, 4)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(44)
+    r = torch.randn(n, device="cuda", generator=gen) * 1e-4
+    g_host, r_host = g.cpu().numpy(), r.cpu().numpy()
+    a = g + r  # fl32(g + r0), the value the step quantizes
+    c = words_like(n)
+    q.cu_fn_matrix_quantize_e(g, c, r, thrd, add_residual=True)
+    c_host = np.empty((n + 15) // 16, dtype=np.uint32)
+    oracle.c.fused_quantize_inplace(g_host, r_host, c_host, thrd)
+    assert_words_equal(host_words(c), c_host)
+    assert torch.equal(r.view(torch.int32), dev(r_host).view(torch.int32)), "residual bits differ"
+    assert c_host.size == 22_176_448
+    # round trip: decode, compare with the oracle's decode, re-quantize the decode -> same codes
+    d = torch.empty(n, device="cuda")
+    q.cu_fn_matrix_dequantize_e(d, c, None, thrd)
+    want_d = oracle.c.dequantize(c_host, n, thrd)
+    assert torch.equal(d.view(torch.int32), dev(want_d).view(torch.int32)), "decode differs"
+    c2, r2 = words_like(n), torch.empty(n, device="cuda")
+    q.cu_fn_matrix_quantize_e(d, c2, r2, thrd)
+    assert torch.equal(c2, c)
+    assert not bool(r2.any())
+    # what was sent plus what is still owed is the input, up to one rounding of the subtraction
+    err = (d.double() + r.double() - a.double()).abs()
+    assert bool((err <= a.double().abs() * 2.0 ** -23).all())
+
+
+def test_config5_hbm_sizing_chunked_error_feedback():
+    """2.8e9 elements resident (11.2 GB gradient + 11.2 GB residual + 0.7 GB codes), N(0, 5e-3),
+    thrd 1e-2, 5 steps in 268,435,456-element chunks.  One whole-vector launch (indices beyond
+    2^31) must equal the chunked result; chunks are checked against the oracle by streaming
+    them through the host: all of them on the first and last step, three per step otherwise."""
+    n, chunk, thrd = 2_800_000_000, 268_435_456, 1e-2
+    starts = list(range(0, n, chunk))
+    assert len(starts) == 11 and n - starts[-1] == 115_645_440
+    g = torch.empty(n, device="cuda")
+    r = torch.zeros(n, device="cuda")
+    c = torch.empty((n + 15) // 16, dtype=torch.int32, device="cuda")
+    gen = torch.Generator(device="cuda")
+    for step in range(5):
+        gen.manual_seed(500 + step)
+        for lo in starts:
+            hi = min(n, lo + chunk)
+            torch.randn(hi - lo, device="cuda", generator=gen, out=g[lo:hi])
+            g[lo:hi].mul_(5e-3)
+        if step == 0:
+            r_whole, c_whole = r.clone(), torch.empty_like(c)
+            q.cu_fn_matrix_quantize_e(g, c_whole, r_whole, thrd, add_residual=True)
+        check = range(len(starts)) if step in (0, 4) else (0, 5, len(starts) - 1)
+        for ci, lo in enumerate(starts):
+            hi = min(n, lo + chunk)
+            verify = ci in check
+            if verify:
+                g_host, r_host = g[lo:hi].cpu().numpy(), r[lo:hi].cpu().numpy()
+            q.cu_fn_matrix_quantize_e(g[lo:hi], c[lo // 16:(hi + 15) // 16], r[lo:hi], thrd,
+                                      add_residual=True, sync=False)
+            if verify:
+                c_host = np.empty((hi - lo + 15) // 16, dtype=np.uint32)
+                oracle.c.fused_quantize_inplace(g_host, r_host, c_host, thrd)
+                assert_words_equal(host_words(c[lo // 16:(hi + 15) // 16]), c_host, f"step {step} chunk {ci}")
+                assert torch.equal(r[lo:hi].view(torch.int32), dev(r_host).view(torch.int32)), \
+                    f"residual differs: step {step} chunk {ci}"
+        torch.cuda.synchronize()
+        if step == 0:
+            assert torch.equal(c_whole, c), "whole-vector launch differs from the chunked result"
+            assert torch.equal(r_whole.view(torch.int32), r.view(torch.int32))
+            del r_whole, c_whole
+    assert int((c != 0).sum()) > 0
