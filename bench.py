@@ -42,7 +42,8 @@ def parse():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--elems", type=int, default=N_ELEMS, help="gradient length (default: the headline size)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU-baseline time budget; 0 skips it")
-    ap.add_argument("--quick", action="store_true", help="skip the extra legs (decode, sum, copy, CPU)")
+    ap.add_argument("--legs", default="deq,acc,copy,cpu",
+                    help="extra legs after the timed quantize steps: deq, acc, copy, cpu (comma list, '' = none)")
     return ap.parse_args()
 
 
@@ -182,8 +183,10 @@ def main():
         },
     }
 
-    if not args.quick:
+    legs = {x for x in args.legs.split(",") if x}
+    if legs & {"deq", "copy"}:
         out = torch.empty(n, dtype=torch.float32, device="cuda")
+    if "deq" in legs:
 
         def deq():
             _lib.check(L.nklq_dequantize_f32(out.data_ptr(), c.data_ptr(), n, 1, THRD, stream))
@@ -199,6 +202,7 @@ def main():
             "frac_hbm_peak": round(BYTES_DEQUANT * n / (deq_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
         }
 
+    if "acc" in legs:
         # receive side at bucket size: 8 payloads (local + 7 synthetic peers, P(0) = 0.9) into one buffer
         nb = 8_000_000 - 3
         wb = _lib.packed_words(nb)
@@ -228,6 +232,7 @@ def main():
             "GBps": round(acc_bytes / (acc_ms * 1e-3) / 1e9, 1),
         }
 
+    if "copy" in legs:
         def cp():
             _lib.check(L.nklq_copy_f32(out.data_ptr(), g.data_ptr(), n, stream))
 
@@ -236,10 +241,10 @@ def main():
         _, ev = time_region(torch, cp, 20)
         res["copy_GBps"] = round(8.0 * n / (ev / 20 * 1e-3) / 1e9, 1)
 
-        if args.cpu_seconds > 0:
-            slab = min(n, 1 << 25)
-            res["cpu_baseline"] = cpu_baseline(g[:slab].cpu().numpy(), r0[:slab].cpu().numpy(),
-                                               args.cpu_seconds)
+    if "cpu" in legs and args.cpu_seconds > 0:
+        slab = min(n, 1 << 25)
+        res["cpu_baseline"] = cpu_baseline(g[:slab].cpu().numpy(), r0[:slab].cpu().numpy(),
+                                           args.cpu_seconds)
     print(json.dumps(res), flush=True)
 
 
