@@ -6,8 +6,8 @@
  * types.  Every pointer marked "device" must be memory the current HIP device
  * can address; `stream` is a hipStream_t passed as an opaque pointer (NULL =
  * the device's default stream).  All entry points are asynchronous on
- * `stream`, allocate nothing, keep no state between calls and may be called
- * from several host threads at once.
+ * `stream`, allocate nothing, keep no state between calls (other than the
+ * nklq_tune knobs) and may be called from several host threads at once.
  *
  * Bit layout (necklace/cuda/quantize.py:8-13, :34-51): codes are 2 bits,
  * 01 = value >= t, 10 = value <= -t, 00 = in between, 16 codes per 32-bit
@@ -116,12 +116,16 @@ int nklq_version(void);
 /*
  * Launch-geometry knobs, the counterpart of the reference wrapper's bpg/tpb
  * keyword arguments (necklace/cuda/quantize.py:98,120).  Results never depend
- * on them.  which: 0 = elements per lane in flight for the flat quantizer
- * (4, 8 or 16), 1 = workgroups per compute unit for the streaming kernels
- * (0 = one workgroup per tile, no grid-stride loop), 2 = non-temporal
- * loads/stores (0/1).  Returns the previous value, or NKLQ_ERANGE.
- * value < 0 only queries.
+ * on them; they apply to the flat kernels of every later call in the process.
+ * Returns the previous value, or NKLQ_ERANGE for an unknown knob or a value
+ * outside its set.  value < 0 only queries.
  */
+#define NKLQ_TUNE_CHUNKS_PER_WAVE 0      /* 256-element chunks per wave: 1, 2 or 4 */
+#define NKLQ_TUNE_WORKGROUP_SIZE 1       /* threads per workgroup: 64, 128, 256, 512 or 1024 */
+#define NKLQ_TUNE_NONTEMPORAL 2          /* non-temporal loads and stores of the fp32 streams: 0 or 1 */
+#define NKLQ_TUNE_XCD_INTERLEAVE_LOG2 3  /* quantize: neighbouring chunks are dealt to 2^v consecutive
+                                            workgroups (which run on different XCDs): 0..6 */
+#define NKLQ_TUNE_XCD_INTERLEAVE_LOG2_DECODE 4  /* the same for dequantize / accumulate */
 int nklq_tune(int which, int value);
 
 /*

@@ -71,7 +71,9 @@ def packed_words(n_rows, n_cols=1):
     return int(lib().nklq_packed_words(n_rows, n_cols))
 
 
-TUNE_ELEMS_PER_LANE, TUNE_WG_PER_CU, TUNE_NONTEMPORAL = 0, 1, 2
+TUNE_CHUNKS_PER_WAVE, TUNE_WORKGROUP_SIZE, TUNE_NONTEMPORAL = 0, 1, 2
+TUNE_XCD_INTERLEAVE_LOG2, TUNE_XCD_INTERLEAVE_LOG2_DECODE = 3, 4
+N_TUNE = 5
 
 
 def tune(which, value=-1):

@@ -68,7 +68,8 @@ def test_argument_errors_are_reported_without_a_launch():
 
 
 def test_tune_knobs_round_trip():
-    for which, good, bad in ((0, (4, 8, 16), 5), (1, (0, 8, 32), 5000), (2, (0, 1), None)):
+    for which, good, bad in ((0, (1, 2, 4), 3), (1, (64, 128, 256, 512, 1024), 96), (2, (0, 1), None),
+                             (3, (0, 1, 2, 3, 4, 5, 6), 7), (4, (0, 3, 6), 7)):
         before = _lib.tune(which)
         for v in good:
             _lib.tune(which, v)

@@ -20,12 +20,14 @@ FLAT_SIZES = list(range(1, 50)) + [63, 64, 65, 255, 256, 257, 1023, 1024, 1025, 
 
 def _knobs():
     """Launch geometries to run every flat test under; results must not depend on them."""
-    return [(16, 0, 1), (8, 0, 0), (4, 2, 1), (16, 1, 0), (16, 8, 1)]
+    default = tuple(_lib.tune(i) for i in range(_lib.N_TUNE))
+    return [default, (1, 64, 1, 3, 1), (2, 128, 0, 0, 2), (4, 256, 1, 3, 3), (4, 1024, 0, 5, 6),
+            (2, 512, 1, 6, 0), (1, 1024, 1, 1, 4)]
 
 
-@pytest.fixture(params=_knobs(), ids=lambda k: f"epl{k[0]}-wg{k[1]}-nt{k[2]}")
+@pytest.fixture(params=_knobs(), ids=lambda k: f"u{k[0]}-wg{k[1]}-nt{k[2]}-x{k[3]}-xd{k[4]}")
 def knobs(request):
-    old = [_lib.tune(i) for i in range(3)]
+    old = [_lib.tune(i) for i in range(_lib.N_TUNE)]
     for i, v in enumerate(request.param):
         _lib.tune(i, v)
     yield request.param
