@@ -1,0 +1,252 @@
+"""Trainer-side buffers and steps for 2-bit compressed gradient exchange.
+
+necklace's trainer prepares gradient compression with
+
+    grd_resi, grd_recv, grd_comp, grd_cmps = mxprms.init_grads_compression(
+        params, kn, grd_siz_thrd=...)                  (necklace/trainer/tnopmx.py:135-151)
+    mxprms.grads_do_nccl(params, prm_recvs, nc, kn, grad_comp_cfg=cfg)   (:334-337)
+
+but the module behind those calls is not in the reference tree, and the PyTorch
+trainers only pass ``grad_comp_cfg`` along without using it
+(necklace/frmwrk/pytorch/ptprms.py:319-401).  This module is that missing piece
+for PyTorch-ROCm, laid out for one big GPU: ONE flat residual buffer, ONE flat
+buffer of packed codes (the payload a rank sends) and ONE ``[kn, words]``
+receive buffer (what an all-gather of the payloads fills), with per-parameter
+views into them.  Every compressed parameter starts on a word boundary, so the
+whole payload is exchanged as a single contiguous ``uint32`` message.
+
+Steps (all on the GPU, through the kernels of libnklq.so):
+
+    compress      a = grad + resi; codes -> comp; resi <- a - decode(codes)
+    exchange      (caller's all-gather of `comp` into `recv`; not part of this module —
+                   with one GPU the peers' slots are filled by the caller)
+    decompress    grad <- sum over ranks, in rank order, of decode(recv[k]);  / kn
+
+Semantics that the reference leaves open and this module fixes: error feedback
+is an fp32 add before quantizing; the sum over ranks is a strict left-to-right
+fp32 sum in rank order (fp32 sums of {0, +t, -t} depend on the order).
+"""
+import torch
+
+from ...cuda import quantize as _q
+
+CMP_RATIO = _q.CMP_RATIO
+DEFAULT_SIZE_THRESHOLD = 1001  # grad_size_threshold default, necklace/trainer/tnopmx.py:137
+DEFAULT_COMP_THRESHOLD = 0.5   # grad_comp_threshold default, necklace/trainer/tnopmx.py:138
+DEFAULT_CHUNK = 268_435_456    # elements per launch of the chunked driver (1 GiB of fp32)
+
+
+def _sync(device, stream):
+    if stream is None:
+        torch.cuda.current_stream(device).synchronize()
+    else:
+        stream.synchronize()
+
+
+def _numel(p):
+    if isinstance(p, int):
+        return p
+    if isinstance(p, torch.Tensor):
+        return p.numel()
+    return p.data.numel() if hasattr(p, "data") else int(p)
+
+
+class GradCompLayout:
+    """Which parameters are compressed and where their residual / code words live.
+
+    Parameters with fewer than `size_threshold` elements are left alone (the
+    reference's ``grad_size_threshold``); the others get consecutive slices of the
+    flat residual (elements) and of the flat payload (words, ceil(numel/16) each).
+    Slices start at multiples of 64 elements / 4 words, so every view is 16-byte
+    aligned inside its buffer; the padding words stay zero.
+    """
+    ELEM_ALIGN = 64
+    WORD_ALIGN = 4
+
+    def __init__(self, numels, size_threshold=DEFAULT_SIZE_THRESHOLD):
+        self.numels = [int(n) for n in numels]
+        self.size_threshold = int(size_threshold)
+        self.compressed = [n >= self.size_threshold and n > 0 for n in self.numels]
+        self.elem_offset, self.word_offset, self.words = [], [], []
+        eo = wo = 0
+        for n, c in zip(self.numels, self.compressed):
+            w = _q.packed_rows(n) if c else 0
+            self.elem_offset.append(eo if c else None)
+            self.word_offset.append(wo if c else None)
+            self.words.append(w)
+            if c:
+                eo = -(-(eo + n) // self.ELEM_ALIGN) * self.ELEM_ALIGN
+                wo = -(-(wo + w) // self.WORD_ALIGN) * self.WORD_ALIGN
+        self.total_elems, self.total_words = eo, wo
+
+    def __len__(self):
+        return len(self.numels)
+
+
+class GradCompressor:
+    """Flat buffers + the compress / decompress steps for one model replica."""
+
+    def __init__(self, params, kn, thrd=DEFAULT_COMP_THRESHOLD, size_threshold=DEFAULT_SIZE_THRESHOLD,
+                 device="cuda", rank=0):
+        if kn < 1:
+            raise ValueError("kn (number of workers) must be >= 1")
+        if not 0 <= rank < kn:
+            raise ValueError("rank must be in [0, kn)")
+        self.kn, self.rank, self.thrd = int(kn), int(rank), float(thrd)
+        self.layout = GradCompLayout([_numel(p) for p in params], size_threshold)
+        lay = self.layout
+        self.device = torch.device(device)
+        self.resi = torch.zeros(lay.total_elems, dtype=torch.float32, device=self.device)
+        # slot k of `recv` holds rank k's payload; this rank's own slot doubles as `comp`
+        self.recv = torch.zeros(self.kn, max(lay.total_words, 1), dtype=torch.int32, device=self.device)
+        self.comp = self.recv[self.rank, :lay.total_words]
+        self.grd_cmps = list(lay.compressed)
+        self.grd_resi, self.grd_comp, self.grd_recv = [], [], []
+        for i in range(len(lay)):
+            if lay.compressed[i]:
+                eo, wo, n, w = lay.elem_offset[i], lay.word_offset[i], lay.numels[i], lay.words[i]
+                self.grd_resi.append(self.resi[eo:eo + n])
+                self.grd_comp.append(self.comp[wo:wo + w])
+                self.grd_recv.append(self.recv[:, wo:wo + w])
+            else:
+                self.grd_resi.append(None)
+                self.grd_comp.append(None)
+                self.grd_recv.append(None)
+
+    # ---- send side
+
+    def compress(self, grads, stream=None, sync=False):
+        """Quantize every compressed parameter's gradient with error feedback.
+
+        `grads[i]` is parameter i's gradient (any shape, contiguous fp32 on the GPU);
+        entries of uncompressed parameters are ignored.  One launch per parameter.
+        """
+        if len(grads) != len(self.layout):
+            raise ValueError(f"expected {len(self.layout)} gradients, got {len(grads)}")
+        for i, g in enumerate(grads):
+            if self.grd_cmps[i] and g.numel() != self.layout.numels[i]:
+                raise ValueError(f"gradient {i}: {g.numel()} elements, layout has {self.layout.numels[i]}")
+        for i, g in enumerate(grads):
+            if not self.grd_cmps[i]:
+                continue
+            _q.cu_fn_matrix_quantize_e(g.reshape(-1), self.grd_comp[i], self.grd_resi[i], self.thrd,
+                                       stream=stream, add_residual=True, sync=False)
+        if sync:
+            _sync(self.device, stream)
+
+    def compress_flat(self, flat_grad, stream=None, sync=False, chunk=DEFAULT_CHUNK):
+        """Quantize one flat gradient buffer that holds exactly the compressed parameters back to
+        back (e.g. a flattened bucket): a single launch, or one per `chunk` elements.
+
+        The packing is then that of ONE flat vector (words do not restart at parameter
+        boundaries); use it with a layout of a single entry per bucket.
+        """
+        idx = [i for i, c in enumerate(self.grd_cmps) if c]
+        if len(idx) != 1:
+            raise ValueError("compress_flat needs a layout with exactly one compressed entry (the bucket)")
+        if flat_grad.numel() != self.layout.numels[idx[0]]:
+            raise ValueError("flat gradient length does not match the layout")
+        quantize_chunked(flat_grad.reshape(-1), self.grd_comp[idx[0]], self.grd_resi[idx[0]], self.thrd,
+                         chunk=chunk, stream=stream, add_residual=True, sync=sync)
+
+    # ---- receive side
+
+    def decompress_sum(self, outs, average=True, stream=None, sync=False):
+        """outs[i] <- sum over ranks k = 0..kn-1 (in that order) of decode(recv[k] of parameter i),
+        divided by kn when `average` (the `/ kn` of necklace/frmwrk/pytorch/ptprms.py:294)."""
+        if len(outs) != len(self.layout):
+            raise ValueError(f"expected {len(self.layout)} outputs, got {len(outs)}")
+        for i, o in enumerate(outs):
+            if not self.grd_cmps[i]:
+                continue
+            if not o.is_contiguous() or o.numel() != self.layout.numels[i]:
+                raise ValueError(f"output {i} must be contiguous with {self.layout.numels[i]} elements")
+            flat = o.view(-1)
+            _q.cu_fn_dequantize_accumulate_e(flat, self.grd_recv[i], self.thrd, accumulate=False,
+                                             stream=stream, sync=False)
+            if average and self.kn > 1:
+                if stream is None:
+                    flat.div_(self.kn)
+                else:
+                    with torch.cuda.stream(stream):
+                        flat.div_(self.kn)
+        if sync:
+            _sync(self.device, stream)
+
+    def state_dict(self):
+        """Error-feedback state that has to survive a restart."""
+        return {"resi": self.resi, "thrd": self.thrd, "numels": list(self.layout.numels),
+                "size_threshold": self.layout.size_threshold}
+
+    def load_state_dict(self, state):
+        if list(state["numels"]) != self.layout.numels or state["size_threshold"] != self.layout.size_threshold:
+            raise ValueError("residual state belongs to a different parameter layout")
+        self.resi.copy_(state["resi"])
+        self.thrd = float(state["thrd"])
+
+
+def quantize_chunked(g, c, r, thrd, chunk=DEFAULT_CHUNK, stream=None, add_residual=True, sync=True):
+    """Quantize a long flat vector in launches of `chunk` elements (a multiple of 16, so the
+    words of consecutive chunks abut and the result equals a single launch over the whole vector)."""
+    if chunk <= 0 or chunk % CMP_RATIO:
+        raise ValueError("chunk must be a positive multiple of 16")
+    if g.dim() != 1 or r.shape != g.shape:
+        raise ValueError("g and r must be flat vectors of the same length")
+    n = g.shape[0]
+    if c.dim() != 1 or c.shape[0] != _q.packed_rows(n):
+        raise ValueError(f"c must hold {_q.packed_rows(n)} words")
+    for lo in range(0, n, chunk):
+        hi = min(n, lo + chunk)
+        _q.cu_fn_matrix_quantize_e(g[lo:hi], c[lo // CMP_RATIO:_q.packed_rows(hi)], r[lo:hi], thrd,
+                                   stream=stream, add_residual=add_residual, sync=False)
+    if sync and n:
+        _sync(g.device, stream)
+
+
+# --------------------------------------------------------------------------- functional surface
+
+def init_grads_compression(params, kn, grd_siz_thrd=DEFAULT_SIZE_THRESHOLD, device="cuda", rank=0,
+                           thrd=DEFAULT_COMP_THRESHOLD):
+    """Counterpart of the call at necklace/trainer/tnopmx.py:140-143.
+
+    Returns ``(grd_resi, grd_recv, grd_comp, grd_cmps)``: per-parameter residuals,
+    ``[kn, words]`` receive slots, local packed codes (views of this rank's receive slot), and
+    which parameters are compressed.  The views keep the flat buffers alive; use
+    `init_grad_comp_cfg` to also get the `GradCompressor` that owns them.
+    """
+    gc = GradCompressor(params, kn, thrd=thrd, size_threshold=grd_siz_thrd, device=device, rank=rank)
+    return gc.grd_resi, gc.grd_recv, gc.grd_comp, gc.grd_cmps
+
+
+def init_grad_comp_cfg(params, kn, grad_comp_cfg=None, device="cuda", rank=0):
+    """Fill a ``grad_comp_cfg`` dict the way TrainerOPMxnet.init_grads_comp does
+    (necklace/trainer/tnopmx.py:135-151): keys grd_resi, grd_recv, grd_comp, grd_cmps,
+    grad_size_threshold, grad_comp_threshold; plus 'compressor', the object that owns the buffers."""
+    cfg = dict(grad_comp_cfg or {})
+    siz = cfg.get("grad_size_threshold", DEFAULT_SIZE_THRESHOLD)
+    thr = cfg.get("grad_comp_threshold", DEFAULT_COMP_THRESHOLD)
+    gc = GradCompressor(params, kn, thrd=thr, size_threshold=siz, device=device, rank=rank)
+    cfg.update(grd_resi=gc.grd_resi, grd_recv=gc.grd_recv, grd_comp=gc.grd_comp, grd_cmps=gc.grd_cmps,
+               grad_size_threshold=siz, grad_comp_threshold=thr, compressor=gc)
+    return cfg
+
+
+def grads_do_compressed_exchange(grads, kn, grad_comp_cfg, exchange=None, average=True, stream=None):
+    """The compressed form of the gradient all-reduce (what ``grads_do_nccl(..., grad_comp_cfg=)``
+    stands for at necklace/trainer/tnopmx.py:334-337): compress, exchange, decompress-sum in place.
+
+    `exchange(comp, recv)` must fill ``recv[k]`` with rank k's payload for all k (an all-gather of
+    `comp`); it is the caller's, since collectives are not part of this module.  With ``kn == 1``
+    it may be omitted.  Returns the indices of the parameters that were NOT compressed and still
+    need the ordinary fp32 all-reduce.
+    """
+    gc = grad_comp_cfg["compressor"]
+    if gc.kn != kn:
+        raise ValueError(f"grad_comp_cfg was built for kn={gc.kn}, got kn={kn}")
+    gc.compress(grads, stream=stream)
+    if exchange is not None:
+        exchange(gc.comp, gc.recv)
+    elif kn != 1:
+        raise ValueError("an exchange callable is required when kn > 1")
+    gc.decompress_sum(grads, average=average, stream=stream)
+    return [i for i, c in enumerate(gc.grd_cmps) if not c]

@@ -1,0 +1,94 @@
+"""Trainer-side compression buffers on the GPU: per-parameter compress with error feedback,
+synthetic peers, fixed-order decompress-sum, chunked driver — all against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from conftest import assert_bits_equal, assert_words_equal
+from gpu_util import dev, host_words, random_payloads_gpu, resnet50_segment_sizes
+from necklace_amd.frmwrk.pytorch import ptcomp
+
+pytestmark = pytest.mark.gpu
+
+
+def test_per_parameter_compress_exchange_decompress_three_steps():
+    """A ResNet-50-shaped set of 161 gradients, kn = 4 (this rank is 1, three synthetic peers),
+    grad_size_threshold 1001: small tensors are skipped, the others go through
+    compress -> exchange -> decompress-sum, three steps with the residual carried."""
+    sizes = resnet50_segment_sizes()
+    kn, rank, thrd = 4, 1, 1e-3
+    cfg = ptcomp.init_grad_comp_cfg(sizes, kn, {"grad_comp_threshold": thrd}, rank=rank)
+    gc = cfg["compressor"]
+    lay = gc.layout
+    assert sum(cfg["grd_cmps"]) == sum(1 for s in sizes if s >= 1001)
+    resid_host = [np.zeros(s, np.float32) for s in sizes]
+    rng = np.random.default_rng(8)
+    sig = 10.0 ** rng.uniform(-4, -2, len(sizes))
+    for step in range(3):
+        grads_host = [(rng.standard_normal(s, dtype=np.float32) * np.float32(sig[i])) for i, s in enumerate(sizes)]
+        grads = [dev(g) for g in grads_host]
+        peers = random_payloads_gpu(kn, 16 * lay.total_words, 900 + step)  # [kn, total_words]
+
+        def exchange(comp, recv, peers=peers):
+            mine = comp.clone()
+            recv.copy_(peers)
+            recv[rank].copy_(mine)
+
+        left = ptcomp.grads_do_compressed_exchange(grads, kn, cfg, exchange=exchange, average=True)
+        assert left == [i for i, s in enumerate(sizes) if s < 1001]
+        torch.cuda.synchronize()
+        peers_host = host_words(peers)
+        for i, s in enumerate(sizes):
+            if s < 1001:
+                assert_bits_equal(grads[i].cpu().numpy(), grads_host[i], f"uncompressed {i} must be untouched")
+                continue
+            want_c, want_r = oracle.c.quantize(grads_host[i], thrd, R_in=resid_host[i])
+            resid_host[i] = want_r
+            wo, w = lay.word_offset[i], lay.words[i]
+            assert_words_equal(host_words(gc.grd_comp[i]), want_c, f"step {step} param {i} codes")
+            assert_bits_equal(gc.grd_resi[i].cpu().numpy(), want_r, f"step {step} param {i} residual")
+            pl = [peers_host[k, wo:wo + w].copy() for k in range(kn)]
+            pl[rank] = want_c
+            want = (oracle.c.dequant_accumulate(pl, s, thrd) / np.float32(kn)).astype(np.float32)
+            assert_bits_equal(grads[i].cpu().numpy(), want, f"step {step} param {i} sum")
+
+
+def test_bucket_compress_flat_and_chunked_driver():
+    n, thrd = 3_000_000 + 7, 5e-3
+    rng = np.random.default_rng(17)
+    g = rng.normal(0, 5e-3, n).astype(np.float32)
+    gc = ptcomp.GradCompressor([n], kn=1, thrd=thrd)
+    r0 = rng.normal(0, 1e-3, n).astype(np.float32)
+    gc.grd_resi[0].copy_(dev(r0))
+    want_c, want_r = oracle.c.quantize(g, thrd, R_in=r0)
+    gc.compress_flat(dev(g), chunk=1 << 20, sync=True)  # three chunks, the last one ragged
+    assert_words_equal(host_words(gc.grd_comp[0]), want_c)
+    assert_bits_equal(gc.grd_resi[0].cpu().numpy(), want_r)
+    out = torch.empty(n, device="cuda")
+    gc.decompress_sum([out], sync=True)
+    assert_bits_equal(out.cpu().numpy(), oracle.c.dequant_accumulate([want_c], n, thrd))
+    # chunked driver on its own buffers equals one launch
+    c1 = torch.full(((n + 15) // 16,), -1, dtype=torch.int32, device="cuda")
+    r1 = dev(r0)
+    ptcomp.quantize_chunked(dev(g), c1, r1, thrd, chunk=4096)
+    assert_words_equal(host_words(c1), want_c)
+    assert_bits_equal(r1.cpu().numpy(), want_r)
+
+
+def test_residual_state_survives_a_restart():
+    n, thrd = 50_000, 1e-3
+    rng = np.random.default_rng(23)
+    gs = [rng.normal(0, 1e-3, n).astype(np.float32) for _ in range(4)]
+    a = ptcomp.GradCompressor([n], kn=1, thrd=thrd)
+    for g in gs[:2]:
+        a.compress([dev(g)])
+    state = {k: (v.clone() if isinstance(v, torch.Tensor) else v) for k, v in a.state_dict().items()}
+    b = ptcomp.GradCompressor([n], kn=1, thrd=thrd)
+    b.load_state_dict(state)
+    for g in gs[2:]:
+        a.compress([dev(g)])
+        b.compress([dev(g)], sync=True)
+    torch.cuda.synchronize()
+    assert torch.equal(a.resi.view(torch.int32), b.resi.view(torch.int32))
+    assert torch.equal(a.comp, b.comp)
