@@ -219,38 +219,23 @@ __global__ __launch_bounds__(BLOCK) void quant_flat_kernel(
     }
 }
 
-// ---------------------------------------------------------------- flat dequantize / accumulate
+// ---------------------------------------------------------------- flat dequantize
 
-struct PayloadPtrs {
-    const uint32_t* p[NKLQ_MAX_PAYLOADS_PER_LAUNCH];
-};
-
-// OVERWRITE: out[j] = decode(payload 0)[j]  (the reference dequantize, flat).
-// otherwise: out[j] = ((start + d_0[j]) + d_1[j]) + ... strictly in payload
-// order, start = accumulate ? out[j] : +0.0f.  The 4 lanes of a quad read the
-// same code word (one 64 B request per wave and payload) and each takes its byte.
-// Code words are read with ordinary (cached) loads: two chunks share a 128 B
-// line, and non-temporal loads of half lines measure 20-35 % slower here.
-template <int U, int BLOCK, bool ALIGNED, bool NT, bool OVERWRITE>
+// out[j] = decode(c)[j]  (the reference dequantize, flat).  The 4 lanes of a quad read the
+// same code word (one 64 B request per wave) and each takes its byte.  Code words are read
+// with ordinary (cached) loads: two chunks share a 128 B line, and non-temporal loads of half
+// lines measure 20-35 % slower here.
+template <int U, int BLOCK, bool ALIGNED, bool NT>
 __global__ __launch_bounds__(BLOCK) void deq_flat_kernel(
-    float* out, PayloadPtrs pl, int k_payloads, uint64_t n, uint64_t n_chunks, uint32_t has_tail,
-    uint32_t xs, float t, int accumulate)
+    float* out, const uint32_t* __restrict__ c, uint64_t n, uint64_t n_chunks, uint32_t has_tail,
+    uint32_t xs, float t)
 {
     if (has_tail && blockIdx.x == gridDim.x - 1) {
         // tail: one element per lane, bounds-checked
         for (int first = 0; first < kChunk; first += BLOCK) {
             const uint64_t e = n_chunks * kChunk + (uint64_t)(first + threadIdx.x);
-            if ((first + (int)threadIdx.x) < kChunk && e < n) {
-                const uint32_t sh = 2 * (uint32_t)(e & 15);
-                if constexpr (OVERWRITE) {
-                    out[e] = deq_code((pl.p[0][e >> 4] >> sh) & 3u, t);
-                } else {
-                    float s = accumulate ? out[e] : 0.0f;
-                    for (int p = 0; p < k_payloads; ++p)
-                        s = s + deq_code((pl.p[p][e >> 4] >> sh) & 3u, t);
-                    out[e] = s;
-                }
-            }
+            if ((first + (int)threadIdx.x) < kChunk && e < n)
+                out[e] = deq_code((c[e >> 4] >> (2 * (uint32_t)(e & 15))) & 3u, t);
         }
         return;
     }
@@ -261,25 +246,128 @@ __global__ __launch_bounds__(BLOCK) void deq_flat_kernel(
     for (int j = 0; j < U; ++j) {
         const uint64_t ch = chunk_of<U, BLOCK>(blockIdx.x, w, j, xs);
         if (ch >= n_chunks) continue;
-        float* o = out + ch * kChunk + lane * 4;
-        const uint64_t wi = ch * kWordsPerChunk + (lane >> 2);
-        if constexpr (OVERWRITE) {
-            st4<ALIGNED, NT>(o, deq_byte((pl.p[0][wi] >> sh) & 0xFFu, t));
-        } else {
-            f32x4 s = (f32x4)(0.0f);
-            if (accumulate) s = ld4<ALIGNED, NT>(o);
-            int p = 0;
-            for (; p + 4 <= k_payloads; p += 4) {  // 4 loads in flight, adds in order
-                const uint32_t w0 = pl.p[p][wi], w1 = pl.p[p + 1][wi];
-                const uint32_t w2 = pl.p[p + 2][wi], w3 = pl.p[p + 3][wi];
-                s = s + deq_byte((w0 >> sh) & 0xFFu, t);
-                s = s + deq_byte((w1 >> sh) & 0xFFu, t);
-                s = s + deq_byte((w2 >> sh) & 0xFFu, t);
-                s = s + deq_byte((w3 >> sh) & 0xFFu, t);
-            }
-            for (; p < k_payloads; ++p) s = s + deq_byte((pl.p[p][wi] >> sh) & 0xFFu, t);
-            st4<ALIGNED, NT>(o, s);
+        const uint32_t word = c[ch * kWordsPerChunk + (lane >> 2)];
+        st4<ALIGNED, NT>(out + ch * kChunk + lane * 4, deq_byte((word >> sh) & 0xFFu, t));
+    }
+}
+
+// ---------------------------------------------------------------- flat accumulate over payloads
+
+struct PayloadPtrs {
+    const uint32_t* p[NKLQ_MAX_PAYLOADS_PER_LAUNCH];
+};
+
+constexpr int kTile = 1024;        // elements per wave in the accumulate kernel: 64 code words
+constexpr int kLdsLaneStride = 20; // floats per lane in LDS (16 used): keeps b128 accesses off shared banks
+
+// Position in a wave's LDS area of element `idx` (0..1023) of the tile.
+__device__ __forceinline__ int lds_pos(int idx) { return kLdsLaneStride * (idx >> 4) + (idx & 15); }
+
+// 2-bit codes -> 2-bit two's complement multipliers, all 16 fields of a word at once:
+// 00 -> 00 (0), 01 -> 01 (+1), 10 -> 11 (-1), 11 -> 00 (0).  Per field (2 + b0 - b1) is 1..3,
+// so the subtraction never borrows across fields; xor 10 then gives the table above.
+__device__ __forceinline__ uint32_t codes_to_multipliers(uint32_t w)
+{
+    const uint32_t e = (w & 0x55555555u) | 0xAAAAAAAAu;
+    const uint32_t o = (w >> 1) & 0x55555555u;
+    return (e - o) ^ 0xAAAAAAAAu;
+}
+
+// acc[j] = ((start + d_0[j]) + d_1[j]) + ... strictly in payload order, start = accumulate ?
+// acc[j] : +0.0f.  With K payloads the sum costs K decodes and K adds per element, so the
+// layout is chosen for the arithmetic: a lane OWNS one code word of each payload (16 elements),
+// so a wave fetches a payload's 64 words with one coalesced 256 B load, every shift is an
+// immediate, and nothing moves between lanes during the sum.  The 16 running sums of a lane are
+// 64 B apart in memory from its neighbour's, so the tile goes through LDS once on the way out
+// (and once on the way in when accumulating) to turn that into 1 KiB-contiguous stores.
+//
+// FMA: when t is finite and not negative, (+t, -t, 0) is k * t with k in {+1, -1, 0} exactly and
+// fma(k, t, s) rounds s + k*t once, i.e. gives the same bits as s + decode: 3 VALU ops per
+// element and payload instead of 6 with compares and selects (which the K = 8 sum would be bound
+// by).  For any other t (negative, NaN, infinite: 0 * t would not be +0) the select form is used.
+template <int BLOCK, bool ALIGNED, bool NT, bool FMA>
+__global__ __launch_bounds__(BLOCK) void acc_flat_kernel(
+    float* acc, PayloadPtrs pl, int k_payloads, uint64_t n, uint64_t n_tiles, uint32_t has_tail,
+    uint32_t xs, float t, int accumulate)
+{
+    constexpr int WPB = BLOCK / kWave;
+    __shared__ __attribute__((aligned(16))) float lds[WPB][kWave * kLdsLaneStride];
+    if (has_tail && blockIdx.x == gridDim.x - 1) {
+        // tail: fewer than 1024 elements, one per lane and round, bounds-checked
+        for (uint64_t e = n_tiles * kTile + threadIdx.x; e < n; e += BLOCK) {
+            const uint32_t sh = 2 * (uint32_t)(e & 15);
+            float s = accumulate ? acc[e] : 0.0f;
+            for (int p = 0; p < k_payloads; ++p) s = s + deq_code((pl.p[p][e >> 4] >> sh) & 3u, t);
+            acc[e] = s;
         }
+        return;
+    }
+    const int lane = threadIdx.x & (kWave - 1);
+    const uint32_t w = threadIdx.x >> 6;
+    const uint64_t tile = chunk_of<1, BLOCK>(blockIdx.x, w, 0, xs);
+    if (tile >= n_tiles) return;
+    float* my = lds[w];
+    float* o = acc + tile * kTile;
+
+    // every payload's word for this lane, all loads in flight together
+    uint32_t wd[NKLQ_MAX_PAYLOADS_PER_LAUNCH];
+#pragma unroll
+    for (int p = 0; p < NKLQ_MAX_PAYLOADS_PER_LAUNCH; ++p)
+        if (p < k_payloads) wd[p] = pl.p[p][tile * (kTile / 16) + lane];
+
+    float s[16];
+    if (accumulate) {
+        // coalesced read of the running sums, through LDS into the one-word-per-lane layout
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const f32x4 v = ld4<ALIGNED, NT>(o + j * 256 + lane * 4);
+            *reinterpret_cast<f32x4*>(my + lds_pos(j * 256 + lane * 4)) = v;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const f32x4 v = *reinterpret_cast<const f32x4*>(my + kLdsLaneStride * lane + 4 * q);
+            s[4 * q] = v.x; s[4 * q + 1] = v.y; s[4 * q + 2] = v.z; s[4 * q + 3] = v.w;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    } else {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[i] = 0.0f;
+    }
+
+#pragma unroll
+    for (int p = 0; p < NKLQ_MAX_PAYLOADS_PER_LAUNCH; ++p) {
+        if (p < k_payloads) {
+            if constexpr (FMA) {
+                const int m = (int)codes_to_multipliers(wd[p]);
+#pragma unroll
+                for (int i = 0; i < 16; ++i)
+                    s[i] = __builtin_fmaf((float)(int)__builtin_amdgcn_sbfe(m, 2 * i, 2), t, s[i]);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) s[i] = s[i] + deq_code((wd[p] >> (2 * i)) & 3u, t);
+            }
+        }
+    }
+
+    // one-word-per-lane layout -> LDS -> 1 KiB-contiguous stores
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        f32x4 v;
+        v.x = s[4 * q]; v.y = s[4 * q + 1]; v.z = s[4 * q + 2]; v.w = s[4 * q + 3];
+        *reinterpret_cast<f32x4*>(my + kLdsLaneStride * lane + 4 * q) = v;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const f32x4 v = *reinterpret_cast<const f32x4*>(my + lds_pos(j * 256 + lane * 4));
+        st4<ALIGNED, NT>(o + j * 256 + lane * 4, v);
     }
 }
 
@@ -496,22 +584,56 @@ int launch_quant_flat(const float* g, const float* rin, float* rout, uint32_t* c
     return launch_status();
 }
 
-template <int U, int BLOCK, bool OVERWRITE>
-int launch_deq_flat(float* out, const PayloadPtrs& pl, int k, uint64_t n, float t, int accumulate,
-                    hipStream_t s)
+template <int U, int BLOCK>
+int launch_deq_flat(float* out, const uint32_t* c, uint64_t n, float t, hipStream_t s)
 {
     const FlatGrid fg = flat_grid(n, U, BLOCK, g_xcd_shift_decode);
     if (fg.blocks == 0) return NKLQ_ERANGE;
     const bool al = aligned16(out);
     const bool nt = g_nontemporal != 0;
-#define NKLQ_DEQ(AL, NT)                                                                          \
-    hipLaunchKernelGGL((deq_flat_kernel<U, BLOCK, AL, NT, OVERWRITE>), dim3(fg.blocks), dim3(BLOCK), \
-                       0, s, out, pl, k, n, fg.n_chunks, fg.has_tail, fg.xs, t, accumulate)
+#define NKLQ_DEQ(AL, NT)                                                                        \
+    hipLaunchKernelGGL((deq_flat_kernel<U, BLOCK, AL, NT>), dim3(fg.blocks), dim3(BLOCK), 0, s, out, \
+                       c, n, fg.n_chunks, fg.has_tail, fg.xs, t)
     if (al && nt) NKLQ_DEQ(true, true);
     else if (al) NKLQ_DEQ(true, false);
     else if (nt) NKLQ_DEQ(false, true);
     else NKLQ_DEQ(false, false);
 #undef NKLQ_DEQ
+    return launch_status();
+}
+
+// The accumulate kernel works on tiles of 1024 elements, one per wave, 256-thread workgroups.
+int launch_acc_flat(float* acc, const PayloadPtrs& pl, int k, uint64_t n, float t, int accumulate,
+                    hipStream_t s)
+{
+    constexpr int BLOCK = 256;
+    const uint32_t xs = (uint32_t)g_xcd_shift_decode;
+    const uint64_t n_tiles = n / kTile;
+    const uint32_t has_tail = (n_tiles * kTile < n) ? 1u : 0u;
+    const uint64_t per_group = (uint64_t)(BLOCK / kWave) << xs;
+    const uint64_t work = ((n_tiles + per_group - 1) / per_group) << xs;
+    if (work + has_tail > 0x7FFFFFFFull) return NKLQ_ERANGE;
+    const uint32_t blocks = (uint32_t)work + has_tail;
+    const bool al = aligned16(acc);
+    const bool nt = g_nontemporal != 0;
+    // fma(k, t, s) reproduces s + decode only when 0 * t is +0 and k * t is exact: finite t >= +0
+    const uint32_t tbits = __builtin_bit_cast(uint32_t, t);
+    const bool fma_ok = (tbits >> 31) == 0 && (tbits & 0x7F800000u) != 0x7F800000u;
+#define NKLQ_ACC(AL, NT, FMA)                                                                     \
+    hipLaunchKernelGGL((acc_flat_kernel<BLOCK, AL, NT, FMA>), dim3(blocks), dim3(BLOCK), 0, s, acc, \
+                       pl, k, n, n_tiles, has_tail, xs, t, accumulate)
+    const int sel = (al ? 4 : 0) | (nt ? 2 : 0) | (fma_ok ? 1 : 0);
+    switch (sel) {
+        case 7: NKLQ_ACC(true, true, true); break;
+        case 6: NKLQ_ACC(true, true, false); break;
+        case 5: NKLQ_ACC(true, false, true); break;
+        case 4: NKLQ_ACC(true, false, false); break;
+        case 3: NKLQ_ACC(false, true, true); break;
+        case 2: NKLQ_ACC(false, true, false); break;
+        case 1: NKLQ_ACC(false, false, true); break;
+        default: NKLQ_ACC(false, false, false); break;
+    }
+#undef NKLQ_ACC
     return launch_status();
 }
 
@@ -544,11 +666,9 @@ int dispatch_quant_flat(const float* g, const float* rin, float* rout, uint32_t*
 #undef NKLQ_CALL
 }
 
-template <bool OVERWRITE>
-int dispatch_deq_flat(float* out, const PayloadPtrs& pl, int k, uint64_t n, float t, int accumulate,
-                      hipStream_t s)
+int dispatch_deq_flat(float* out, const uint32_t* c, uint64_t n, float t, hipStream_t s)
 {
-#define NKLQ_CALL(U, B) launch_deq_flat<U, B, OVERWRITE>(out, pl, k, n, t, accumulate, s)
+#define NKLQ_CALL(U, B) launch_deq_flat<U, B>(out, c, n, t, s)
     NKLQ_FOR_GEOMETRY(NKLQ_CALL)
 #undef NKLQ_CALL
 }
@@ -703,9 +823,7 @@ int nklq_dequantize_f32(float* out, const uint32_t* c, uint64_t n_rows, uint64_t
     if ((const void*)c == (const void*)out) return NKLQ_EALIAS;
     hipStream_t s = (hipStream_t)stream;
     if (n_cols == 1) {
-        PayloadPtrs pl = {};
-        for (int p = 0; p < NKLQ_MAX_PAYLOADS_PER_LAUNCH; ++p) pl.p[p] = c;
-        return dispatch_deq_flat<true>(out, pl, 1, total, thrd, 0, s);
+        return dispatch_deq_flat(out, c, total, thrd, s);
     }
     const uint64_t m = n_rows / 16 + (n_rows % 16 ? 1 : 0);
     if ((n_cols % 4 == 0) && aligned16(out) && aligned16(c)) {
@@ -740,7 +858,7 @@ int nklq_dequant_accumulate_f32(float* acc, const uint32_t* const* payloads, int
         if (k > NKLQ_MAX_PAYLOADS_PER_LAUNCH) k = NKLQ_MAX_PAYLOADS_PER_LAUNCH;
         for (int p = 0; p < k; ++p) pl.p[p] = payloads[first + p];
         for (int p = k; p < NKLQ_MAX_PAYLOADS_PER_LAUNCH; ++p) pl.p[p] = payloads[first];
-        const int st = dispatch_deq_flat<false>(acc, pl, k, n, thrd, acc_flag, s);
+        const int st = launch_acc_flat(acc, pl, k, n, thrd, acc_flag, s);
         if (st != NKLQ_OK) return st;
         acc_flag = 1;  // later launches continue the running sum held in acc
     }

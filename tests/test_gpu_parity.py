@@ -187,6 +187,36 @@ def test_accumulate_fixed_order(k_payloads, knobs):
         assert_bits_equal(acc2.cpu().numpy(), want2, f"n={n} accumulate")
 
 
+@pytest.mark.parametrize("thrd", [0.0, -0.0, -0.25, 1e-45, 3e38, float("inf"), float("-inf"), float("nan")])
+def test_accumulate_and_decode_with_unusual_thresholds(thrd):
+    """Zero, negative, denormal, huge and non-finite thresholds decode exactly like the reference
+    (the sum then takes the compare-and-select form instead of the fused multiply-add one)."""
+    rng = np.random.default_rng(77)
+    n = 5000 + 11
+    pl = [pack_codes_np(rng.integers(0, 4, size=n).astype(np.uint32), n) for _ in range(5)]
+    base = rng.normal(0, 1, n).astype(np.float32)
+    base[::7] = -0.0
+    for acc0 in (None, base):
+        with np.errstate(invalid="ignore", over="ignore"):
+            want = oracle.c.dequant_accumulate(pl, n, thrd, acc=acc0)
+        acc = torch.full((n,), 5.0, device="cuda") if acc0 is None else dev(acc0)
+        q.cu_fn_dequantize_accumulate_e(acc, [dev(w) for w in pl], thrd, accumulate=acc0 is not None)
+        assert_bits_equal(acc.cpu().numpy(), want, f"thrd={thrd}")
+    assert_bits_equal(gpu_dequantize(pl[0], n, thrd), oracle.c.dequantize(pl[0], n, thrd), f"decode thrd={thrd}")
+
+
+def test_accumulate_keeps_signed_zero_like_the_reference():
+    """-0.0 + (+0.0) is +0.0: an all-zero payload turns a -0.0 running sum into +0.0, on both sides."""
+    n = 2048 + 3
+    zeros = np.zeros((n + 15) // 16, dtype=np.uint32)
+    base = np.full(n, -0.0, dtype=np.float32)
+    want = oracle.c.dequant_accumulate([zeros], n, 1e-3, acc=base)
+    acc = dev(base)
+    q.cu_fn_dequantize_accumulate_e(acc, [dev(zeros)], 1e-3, accumulate=True)
+    assert_bits_equal(acc.cpu().numpy(), want)
+    assert not np.signbit(want).any()
+
+
 def test_round_trip_and_zero_residual_on_gpu():
     rng = np.random.default_rng(21)
     n = 1 << 20

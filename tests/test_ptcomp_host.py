@@ -11,11 +11,11 @@ def test_layout_thresholds_offsets_and_alignment():
     # necklace/trainer/tnopmx.py:137: parameters below grad_size_threshold are not compressed
     assert lay.compressed == [True, False, False, True, False, True, False]
     assert lay.words == [588, 0, 0, 63, 0, 257, 0]
-    assert lay.elem_offset == [0, None, None, 9408, None, 9408 + 1024, None]
-    assert lay.word_offset == [0, None, None, 588, None, 588 + 64, None]
-    assert all(o % 64 == 0 for o in lay.elem_offset if o is not None)
-    assert all(o % 4 == 0 for o in lay.word_offset if o is not None)
-    assert lay.total_elems == 9408 + 1024 + 4160 and lay.total_words == 588 + 64 + 260
+    assert lay.elem_offset == [0, None, None, 9472, None, 9472 + 1024, None]
+    assert lay.word_offset == [0, None, None, 592, None, 592 + 64, None]
+    assert all(o % 256 == 0 for o in lay.elem_offset if o is not None)
+    assert all(o % 16 == 0 for o in lay.word_offset if o is not None)
+    assert lay.total_elems == 9472 + 1024 + 4352 and lay.total_words == 592 + 64 + 272
 
 
 def test_cfg_has_the_keys_the_trainer_stores():
