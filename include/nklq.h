@@ -102,6 +102,30 @@ int nklq_dequant_accumulate_f32(float* acc, const uint32_t* const* payloads, int
                                 uint64_t n, float thrd, int accumulate, void* stream);
 
 /*
+ * The two flat operations above on MANY vectors with one launch per 32 of them: a model's
+ * gradients are a list of separate tensors, and the per-parameter lists grd_resi / grd_comp /
+ * grd_recv that necklace's trainer keeps (necklace/trainer/tnopmx.py:140-149) are lists of
+ * separate buffers.  All array arguments are HOST arrays of `count` entries, read during the
+ * call only.  Vectors with n[i] == 0 are skipped.
+ *
+ * nklq_quantize_multi_f32: for every i the flat quantize of g[i] (n[i] elements) into c[i]
+ * (ceil(n[i]/16) words); the residual r[i] is updated in place when add_residual != 0
+ * (a = g + r) and only written otherwise.
+ *
+ * nklq_dequant_accumulate_multi_f32: for every i the fixed-order sum of nklq_dequant_accumulate_f32
+ * into acc[i], where vector i's code words start at word_offset[i] inside each of the
+ * k_payloads payload buffers payload_base[p] (one contiguous message per peer).  The sum is
+ * divided by `divisor` (IEEE division) before it is stored unless divisor == 1: the `/ kn` that
+ * follows the all-reduce at necklace/frmwrk/pytorch/ptprms.py:294.
+ */
+int nklq_quantize_multi_f32(int count, const float* const* g, float* const* r, uint32_t* const* c,
+                            const uint64_t* n, float thrd, int add_residual, void* stream);
+int nklq_dequant_accumulate_multi_f32(int count, float* const* acc, const uint64_t* n,
+                                      const uint64_t* word_offset,
+                                      const uint32_t* const* payload_base, int k_payloads,
+                                      float thrd, int accumulate, float divisor, void* stream);
+
+/*
  * Number of uint32 words of the packed matrix: ceil(n_rows/16) * n_cols
  * (the `m` of necklace/cuda/quantize.py:145-147 times the column count).
  */

@@ -19,6 +19,7 @@ NKLQ_MAX_PAYLOADS_PER_LAUNCH = 16
 
 SYMBOLS = (
     "nklq_quantize_f32", "nklq_dequantize_f32", "nklq_dequant_accumulate_f32",
+    "nklq_quantize_multi_f32", "nklq_dequant_accumulate_multi_f32",
     "nklq_packed_words", "nklq_strerror", "nklq_version", "nklq_tune", "nklq_copy_f32",
 )
 
@@ -48,6 +49,12 @@ def lib():
     L.nklq_dequantize_f32.restype = i32
     L.nklq_dequant_accumulate_f32.argtypes = [vp, ct.POINTER(vp), i32, u64, f32, i32, vp]
     L.nklq_dequant_accumulate_f32.restype = i32
+    L.nklq_quantize_multi_f32.argtypes = [i32, ct.POINTER(vp), ct.POINTER(vp), ct.POINTER(vp),
+                                          ct.POINTER(u64), f32, i32, vp]
+    L.nklq_quantize_multi_f32.restype = i32
+    L.nklq_dequant_accumulate_multi_f32.argtypes = [i32, ct.POINTER(vp), ct.POINTER(u64), ct.POINTER(u64),
+                                                    ct.POINTER(vp), i32, f32, i32, f32, vp]
+    L.nklq_dequant_accumulate_multi_f32.restype = i32
     L.nklq_packed_words.argtypes = [u64, u64]
     L.nklq_packed_words.restype = u64
     L.nklq_strerror.argtypes = [i32]

@@ -42,7 +42,7 @@ typedef f32x4 f32x4_a4 __attribute__((aligned(4)));
 constexpr int kWave = 64;
 constexpr int kChunk = 256;          // elements per chunk: one dwordx4 per lane
 constexpr int kWordsPerChunk = 16;
-constexpr int kBlock2D = 256;        // workgroup size of the matrix kernels
+constexpr int kBlock2D = 256;        // workgroup size of the general matrix kernels
 
 // ---------------------------------------------------------------- per element
 
@@ -373,109 +373,306 @@ __global__ __launch_bounds__(BLOCK) void acc_flat_kernel(
 
 // ---------------------------------------------------------------- matrix (n, k) kernels
 
-// Word (x, y) packs rows 16x .. 16x+15 of column y (quantize.py:35-51).  Lanes
-// walk along y, the contiguous dimension; VEC columns per lane.
-template <int VEC, bool ADD>
+// Word (x, y) packs rows 16x .. 16x+15 of column y (quantize.py:35-51).
+//
+// General form, any k and any 4-byte-aligned bases: one lane per word, lanes walk along y (the
+// contiguous dimension), so a wave reads 256 B of each of its 16 rows.
+template <bool ADD>
 __global__ __launch_bounds__(kBlock2D) void quant_2d_kernel(
     const float* g, const float* rin, float* rout, uint32_t* __restrict__ c, uint64_t n,
     uint64_t k, uint64_t items, float t)
 {
-    const uint64_t kv = k / VEC;  // lanes per row of words
     for (uint64_t it = (uint64_t)blockIdx.x * kBlock2D + threadIdx.x; it < items;
          it += (uint64_t)gridDim.x * kBlock2D) {
-        const uint64_t x = it / kv;
-        const uint64_t y = (it - x * kv) * VEC;
-        uint32_t w[VEC];
-#pragma unroll
-        for (int v = 0; v < VEC; ++v) w[v] = 0;
+        const uint64_t x = it / k;
+        const uint64_t y = it - x * k;
+        uint32_t word = 0;
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
-            float a[8][VEC];
-            float r[8][VEC];
+            float a[8];
+            float r[8];
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 const uint64_t xm = x * 16 + half * 8 + i;
                 if (xm < n) {
-                    const uint64_t off = xm * k + y;
-                    if constexpr (VEC == 4) {
-                        const f32x4 q = *reinterpret_cast<const f32x4*>(g + off);
-                        a[i][0] = q.x; a[i][1] = q.y; a[i][2] = q.z; a[i][3] = q.w;
-                        if constexpr (ADD) {
-                            const f32x4 p = *reinterpret_cast<const f32x4*>(rin + off);
-                            r[i][0] = p.x; r[i][1] = p.y; r[i][2] = p.z; r[i][3] = p.w;
-                        }
-                    } else {
-                        a[i][0] = g[off];
-                        if constexpr (ADD) r[i][0] = rin[off];
-                    }
+                    a[i] = g[xm * k + y];
+                    if constexpr (ADD) r[i] = rin[xm * k + y];
                 }
             }
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 const uint64_t xm = x * 16 + half * 8 + i;
                 if (xm < n) {
-                    const uint64_t off = xm * k + y;
-                    float o[VEC];
-#pragma unroll
-                    for (int v = 0; v < VEC; ++v) {
-                        float val = a[i][v];
-                        if constexpr (ADD) val = val + r[i][v];
-                        w[v] |= quant_one(val, t, o[v]) << (2 * (half * 8 + i));
-                    }
-                    if constexpr (VEC == 4) {
-                        f32x4 q;
-                        q.x = o[0]; q.y = o[1]; q.z = o[2]; q.w = o[3];
-                        *reinterpret_cast<f32x4*>(rout + off) = q;
-                    } else {
-                        rout[off] = o[0];
-                    }
+                    float val = a[i];
+                    if constexpr (ADD) val = val + r[i];
+                    float o;
+                    word |= quant_one(val, t, o) << (2 * (half * 8 + i));
+                    rout[xm * k + y] = o;
                 }
             }
         }
-        if constexpr (VEC == 4) {
-            u32x4 q;
-            q.x = w[0]; q.y = w[1]; q.z = w[2]; q.w = w[3];
-            *reinterpret_cast<u32x4*>(c + x * k + y) = q;
-        } else {
-            c[x * k + y] = w[0];
-        }
+        c[x * k + y] = word;
     }
 }
 
-template <int VEC>
 __global__ __launch_bounds__(kBlock2D) void deq_2d_kernel(float* out, const uint32_t* __restrict__ c,
                                                            uint64_t n, uint64_t k, uint64_t items,
                                                            float t)
 {
-    const uint64_t kv = k / VEC;
     for (uint64_t it = (uint64_t)blockIdx.x * kBlock2D + threadIdx.x; it < items;
          it += (uint64_t)gridDim.x * kBlock2D) {
-        const uint64_t x = it / kv;
-        const uint64_t y = (it - x * kv) * VEC;
-        uint32_t w[VEC];
-        if constexpr (VEC == 4) {
-            const u32x4 q = *reinterpret_cast<const u32x4*>(c + x * k + y);
-            w[0] = q.x; w[1] = q.y; w[2] = q.z; w[3] = q.w;
-        } else {
-            w[0] = c[x * k + y];
-        }
+        const uint64_t x = it / k;
+        const uint64_t y = it - x * k;
+        const uint32_t word = c[x * k + y];
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             const uint64_t xm = x * 16 + i;
-            if (xm < n) {
-                const uint64_t off = xm * k + y;
-                if constexpr (VEC == 4) {
-                    f32x4 q;
-                    q.x = deq_code((w[0] >> (2 * i)) & 3u, t);
-                    q.y = deq_code((w[1] >> (2 * i)) & 3u, t);
-                    q.z = deq_code((w[2] >> (2 * i)) & 3u, t);
-                    q.w = deq_code((w[3] >> (2 * i)) & 3u, t);
-                    *reinterpret_cast<f32x4*>(out + off) = q;
-                } else {
-                    out[off] = deq_code((w[0] >> (2 * i)) & 3u, t);
-                }
+            if (xm < n) out[xm * k + y] = deq_code((word >> (2 * i)) & 3u, t);
+        }
+    }
+}
+
+// Row-tiled matrix kernels, used when k % 4 == 0 and the bases are 16-byte aligned.  A
+// workgroup of 16 waves takes a tile of 16 rows x 256 columns: wave i moves row 16x+i of the
+// tile with one dwordx4 per lane (1 KiB contiguous, like a flat chunk), so neighbouring
+// workgroups (on different XCDs) touch neighbouring 1 KiB pieces of the same rows.  The 16 codes
+// of a word come from 16 different waves: each wave ORs its code, shifted to its bit position,
+// into the tile's 256 words in LDS; after a barrier 256 threads store the 1 KiB of words.
+constexpr int kRowsBlock = 16 * kWave;  // 1024 threads
+
+template <bool ADD, bool NT>
+__global__ __launch_bounds__(kRowsBlock) void quant_2d_rows_kernel(
+    const float* g, const float* rin, float* rout, uint32_t* __restrict__ c, uint64_t n,
+    uint64_t k, uint32_t col_tiles, float t)
+{
+    __shared__ uint32_t words[256];
+    const int lane = threadIdx.x & (kWave - 1);
+    const uint32_t i = threadIdx.x >> 6;  // row inside the tile = code position inside the word
+    const uint64_t x = blockIdx.x / col_tiles;
+    const uint64_t y0 = (uint64_t)(blockIdx.x % col_tiles) * 256;
+    const uint64_t y = y0 + (uint64_t)lane * 4;
+    const uint64_t row = x * 16 + i;
+    const bool live = row < n && y < k;
+    const uint64_t off = row * k + y;
+    f32x4 a = (f32x4)(0.0f), r = (f32x4)(0.0f);
+    if (live) {
+        a = ld4<true, NT>(g + off);
+        if constexpr (ADD) r = ld4<true, NT>(rin + off);
+    }
+    if (threadIdx.x < 256) words[threadIdx.x] = 0;
+    __syncthreads();
+    if (live) {
+        f32x4 v = a;
+        if constexpr (ADD) v = v + r;
+        float o0, o1, o2, o3;
+        const uint32_t c0 = quant_one(v.x, t, o0), c1 = quant_one(v.y, t, o1);
+        const uint32_t c2 = quant_one(v.z, t, o2), c3 = quant_one(v.w, t, o3);
+        f32x4 o;
+        o.x = o0; o.y = o1; o.z = o2; o.w = o3;
+        st4<true, NT>(rout + off, o);
+        const uint32_t sh = 2 * i;
+        if (c0) atomicOr(&words[lane * 4 + 0], c0 << sh);
+        if (c1) atomicOr(&words[lane * 4 + 1], c1 << sh);
+        if (c2) atomicOr(&words[lane * 4 + 2], c2 << sh);
+        if (c3) atomicOr(&words[lane * 4 + 3], c3 << sh);
+    }
+    __syncthreads();
+    if (threadIdx.x < 256 && y0 + threadIdx.x < k) c[x * k + y0 + threadIdx.x] = words[threadIdx.x];
+}
+
+template <bool NT>
+__global__ __launch_bounds__(kRowsBlock) void deq_2d_rows_kernel(
+    float* out, const uint32_t* __restrict__ c, uint64_t n, uint64_t k, uint32_t col_tiles, float t)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    const uint32_t i = threadIdx.x >> 6;
+    const uint64_t x = blockIdx.x / col_tiles;
+    const uint64_t y = (uint64_t)(blockIdx.x % col_tiles) * 256 + (uint64_t)lane * 4;
+    const uint64_t row = x * 16 + i;
+    if (row >= n || y >= k) return;
+    // all 16 waves read the tile's 1 KiB of words (cache hits after the first)
+    const u32x4 w = *reinterpret_cast<const u32x4*>(c + x * k + y);
+    const uint32_t sh = 2 * i;
+    f32x4 o;
+    o.x = deq_code((w.x >> sh) & 3u, t);
+    o.y = deq_code((w.y >> sh) & 3u, t);
+    o.z = deq_code((w.z >> sh) & 3u, t);
+    o.w = deq_code((w.w >> sh) & 3u, t);
+    st4<true, NT>(out + row * k + y, o);
+}
+
+// ---------------------------------------------------------------- many vectors in one launch
+
+// A model's gradients are many separate vectors (161 for ResNet-50, most of them small); one
+// launch per vector costs more in launch latency than the data takes to stream.  These kernels
+// take a table of up to kMaxSegments vectors in their arguments and treat the chunks (or tiles)
+// of all of them as one index space; a wave finds its vector by binary search in the table.
+
+constexpr int kMaxSegments = 32;
+
+struct QuantSegments {
+    const float* g[kMaxSegments];
+    float* r[kMaxSegments];
+    uint32_t* c[kMaxSegments];
+    uint64_t n[kMaxSegments];
+    uint32_t first[kMaxSegments + 1];  // first[s] = index of segment s's first chunk; first[count] = total
+    int count;
+};
+
+// Largest s with first[s] <= q (q < first[count]).
+__device__ __forceinline__ int find_segment(const uint32_t* first, int count, uint32_t q)
+{
+    int lo = 0, hi = count;  // invariant: first[lo] <= q < first[hi]
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (first[mid] <= q) lo = mid;
+        else hi = mid;
+    }
+    return lo;
+}
+
+template <bool ALIGNED, bool ADD, bool NT>
+__global__ __launch_bounds__(256) void quant_multi_kernel(QuantSegments seg, uint32_t xs, float t)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    const uint32_t w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint64_t q64 = chunk_of<1, 256>(blockIdx.x, w, 0, xs);
+    if (q64 >= seg.first[seg.count]) return;
+    const uint32_t q = (uint32_t)q64;
+    const int sidx = find_segment(seg.first, seg.count, q);
+    const float* g = seg.g[sidx];
+    float* r = seg.r[sidx];
+    uint32_t* c = seg.c[sidx];
+    const uint64_t n = seg.n[sidx];
+    const uint64_t e0 = (uint64_t)(q - seg.first[sidx]) * kChunk;
+    if (e0 + kChunk <= n) {
+        const uint64_t e = e0 + lane * 4;
+        f32x4 v = ld4<ALIGNED, NT>(g + e);
+        if constexpr (ADD) v = v + ld4<ALIGNED, NT>(r + e);
+        float o0, o1, o2, o3;
+        uint32_t b = quant_one(v.x, t, o0);
+        b |= quant_one(v.y, t, o1) << 2;
+        b |= quant_one(v.z, t, o2) << 4;
+        b |= quant_one(v.w, t, o3) << 6;
+        f32x4 o;
+        o.x = o0; o.y = o1; o.z = o2; o.w = o3;
+        st4<ALIGNED, NT>(r + e, o);
+        const uint32_t word = quad_or(b << (8 * (lane & 3)));
+        if ((lane & 3) == 0) c[(e0 >> 4) + (lane >> 2)] = word;
+    } else {
+        // last, partial chunk of the vector: one element per lane, 4 rounds, all lanes reach row_or
+#pragma unroll
+        for (int first = 0; first < kChunk; first += kWave) {
+            const uint64_t e = e0 + (uint64_t)(first + lane);
+            const bool live = e < n;
+            uint32_t code = 0;
+            if (live) {
+                float a = g[e];
+                if constexpr (ADD) a = a + r[e];
+                float res;
+                code = quant_one(a, t, res);
+                r[e] = res;
+            }
+            const uint32_t word = row_or(code << (2 * (lane & 15)));
+            if (live && (lane & 15) == 0) c[e >> 4] = word;
+        }
+    }
+}
+
+struct AccSegments {
+    float* acc[kMaxSegments];
+    uint64_t n[kMaxSegments];
+    uint64_t word_offset[kMaxSegments];  // of the vector's first code word inside every payload
+    uint32_t first[kMaxSegments + 1];    // in tiles of 1024 elements
+    int count;
+};
+
+template <bool ALIGNED, bool NT, bool FMA>
+__global__ __launch_bounds__(256) void acc_multi_kernel(AccSegments seg, PayloadPtrs pl, int k_payloads,
+                                                        uint32_t xs, float t, int accumulate,
+                                                        float divisor)
+{
+    const bool divide = divisor != 1.0f;  // IEEE division, correctly rounded (not a reciprocal)
+    __shared__ __attribute__((aligned(16))) float lds[4][kWave * kLdsLaneStride];
+    const int lane = threadIdx.x & (kWave - 1);
+    const uint32_t w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint64_t q64 = chunk_of<1, 256>(blockIdx.x, w, 0, xs);
+    if (q64 >= seg.first[seg.count]) return;
+    const uint32_t q = (uint32_t)q64;
+    const int sidx = find_segment(seg.first, seg.count, q);
+    const uint64_t n = seg.n[sidx];
+    const uint64_t e0 = (uint64_t)(q - seg.first[sidx]) * kTile;
+    float* o = seg.acc[sidx] + e0;
+    const uint64_t w0 = seg.word_offset[sidx] + (e0 >> 4);
+    if (e0 + kTile > n) {
+        // last, partial tile of the vector: one element per lane and round, bounds-checked
+        for (uint64_t e = e0 + lane; e < n; e += kWave) {
+            const uint32_t sh = 2 * (uint32_t)(e & 15);
+            float s = accumulate ? seg.acc[sidx][e] : 0.0f;
+            for (int p = 0; p < k_payloads; ++p)
+                s = s + deq_code((pl.p[p][seg.word_offset[sidx] + (e >> 4)] >> sh) & 3u, t);
+            seg.acc[sidx][e] = divide ? s / divisor : s;
+        }
+        return;
+    }
+    float* my = lds[w];
+    uint32_t wd[NKLQ_MAX_PAYLOADS_PER_LAUNCH];
+#pragma unroll
+    for (int p = 0; p < NKLQ_MAX_PAYLOADS_PER_LAUNCH; ++p)
+        if (p < k_payloads) wd[p] = pl.p[p][w0 + lane];
+    float s[16];
+    if (accumulate) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const f32x4 v = ld4<ALIGNED, NT>(o + j * 256 + lane * 4);
+            *reinterpret_cast<f32x4*>(my + lds_pos(j * 256 + lane * 4)) = v;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int qd = 0; qd < 4; ++qd) {
+            const f32x4 v = *reinterpret_cast<const f32x4*>(my + kLdsLaneStride * lane + 4 * qd);
+            s[4 * qd] = v.x; s[4 * qd + 1] = v.y; s[4 * qd + 2] = v.z; s[4 * qd + 3] = v.w;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    } else {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[i] = 0.0f;
+    }
+#pragma unroll
+    for (int p = 0; p < NKLQ_MAX_PAYLOADS_PER_LAUNCH; ++p) {
+        if (p < k_payloads) {
+            if constexpr (FMA) {
+                const int m = (int)codes_to_multipliers(wd[p]);
+#pragma unroll
+                for (int i = 0; i < 16; ++i)
+                    s[i] = __builtin_fmaf((float)(int)__builtin_amdgcn_sbfe(m, 2 * i, 2), t, s[i]);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) s[i] = s[i] + deq_code((wd[p] >> (2 * i)) & 3u, t);
             }
         }
+    }
+    if (divide) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[i] = s[i] / divisor;
+    }
+#pragma unroll
+    for (int qd = 0; qd < 4; ++qd) {
+        f32x4 v;
+        v.x = s[4 * qd]; v.y = s[4 * qd + 1]; v.z = s[4 * qd + 2]; v.w = s[4 * qd + 3];
+        *reinterpret_cast<f32x4*>(my + kLdsLaneStride * lane + 4 * qd) = v;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const f32x4 v = *reinterpret_cast<const f32x4*>(my + lds_pos(j * 256 + lane * 4));
+        st4<ALIGNED, NT>(o + j * 256 + lane * 4, v);
     }
 }
 
@@ -694,6 +891,66 @@ int dispatch_copy(float* dst, const float* src, uint64_t n, hipStream_t s)
 #undef NKLQ_CALL
 }
 
+// Workgroups for `total` wave items (chunks or tiles), 4 waves per workgroup, dealt over 2^xs.
+bool multi_grid(uint64_t total, uint32_t xs, uint32_t* blocks)
+{
+    const uint64_t per_group = (uint64_t)4 << xs;
+    const uint64_t work = ((total + per_group - 1) / per_group) << xs;
+    if (work > 0x7FFFFFFFull) return false;
+    *blocks = (uint32_t)work;
+    return true;
+}
+
+int launch_quant_multi(const QuantSegments& seg, bool al, bool add, float t, hipStream_t s)
+{
+    uint32_t blocks;
+    const uint32_t xs = (uint32_t)g_xcd_shift;
+    if (!multi_grid(seg.first[seg.count], xs, &blocks)) return NKLQ_ERANGE;
+    if (blocks == 0) return NKLQ_OK;
+    const bool nt = g_nontemporal != 0;
+#define NKLQ_QM(AL, ADD, NT) \
+    hipLaunchKernelGGL((quant_multi_kernel<AL, ADD, NT>), dim3(blocks), dim3(256), 0, s, seg, xs, t)
+    switch ((al ? 4 : 0) | (add ? 2 : 0) | (nt ? 1 : 0)) {
+        case 7: NKLQ_QM(true, true, true); break;
+        case 6: NKLQ_QM(true, true, false); break;
+        case 5: NKLQ_QM(true, false, true); break;
+        case 4: NKLQ_QM(true, false, false); break;
+        case 3: NKLQ_QM(false, true, true); break;
+        case 2: NKLQ_QM(false, true, false); break;
+        case 1: NKLQ_QM(false, false, true); break;
+        default: NKLQ_QM(false, false, false); break;
+    }
+#undef NKLQ_QM
+    return launch_status();
+}
+
+int launch_acc_multi(const AccSegments& seg, const PayloadPtrs& pl, int k, bool al, float t,
+                     int accumulate, float divisor, hipStream_t s)
+{
+    uint32_t blocks;
+    const uint32_t xs = (uint32_t)g_xcd_shift_decode;
+    if (!multi_grid(seg.first[seg.count], xs, &blocks)) return NKLQ_ERANGE;
+    if (blocks == 0) return NKLQ_OK;
+    const bool nt = g_nontemporal != 0;
+    const uint32_t tbits = __builtin_bit_cast(uint32_t, t);
+    const bool fma_ok = (tbits >> 31) == 0 && (tbits & 0x7F800000u) != 0x7F800000u;
+#define NKLQ_AM(AL, NT, FMA)                                                                      \
+    hipLaunchKernelGGL((acc_multi_kernel<AL, NT, FMA>), dim3(blocks), dim3(256), 0, s, seg, pl, k, xs, \
+                       t, accumulate, divisor)
+    switch ((al ? 4 : 0) | (nt ? 2 : 0) | (fma_ok ? 1 : 0)) {
+        case 7: NKLQ_AM(true, true, true); break;
+        case 6: NKLQ_AM(true, true, false); break;
+        case 5: NKLQ_AM(true, false, true); break;
+        case 4: NKLQ_AM(true, false, false); break;
+        case 3: NKLQ_AM(false, true, true); break;
+        case 2: NKLQ_AM(false, true, false); break;
+        case 1: NKLQ_AM(false, false, true); break;
+        default: NKLQ_AM(false, false, false); break;
+    }
+#undef NKLQ_AM
+    return launch_status();
+}
+
 uint32_t grid_for_items(uint64_t items)
 {
     uint64_t blocks = (items + kBlock2D - 1) / kBlock2D;
@@ -791,22 +1048,29 @@ int nklq_quantize_f32(const float* g, const float* r_in, float* r_out, uint32_t*
     const bool vec = (n_cols % 4 == 0) && aligned16(g) && aligned16(r_out) && aligned16(c) &&
                      (!add || aligned16(r_in));
     if (vec) {
-        const uint64_t items = m * (n_cols / 4);
-        const uint32_t grid = grid_for_items(items);
-        if (add)
-            hipLaunchKernelGGL((quant_2d_kernel<4, true>), dim3(grid), dim3(kBlock2D), 0, s, g, r_in,
-                               r_out, c, n_rows, n_cols, items, thrd);
-        else
-            hipLaunchKernelGGL((quant_2d_kernel<4, false>), dim3(grid), dim3(kBlock2D), 0, s, g, r_in,
-                               r_out, c, n_rows, n_cols, items, thrd);
+        const uint64_t col_tiles = (n_cols + 255) / 256;
+        const uint64_t tiles = m * col_tiles;
+        if (tiles > 0x7FFFFFFFull || col_tiles > 0xFFFFFFFFull) return NKLQ_ERANGE;
+        const dim3 grid((uint32_t)tiles), block(kRowsBlock);
+        const int sel = (add ? 2 : 0) | (g_nontemporal ? 1 : 0);
+#define NKLQ_Q2(ADD, NT)                                                                        \
+    hipLaunchKernelGGL((quant_2d_rows_kernel<ADD, NT>), grid, block, 0, s, g, r_in, r_out, c, n_rows, \
+                       n_cols, (uint32_t)col_tiles, thrd)
+        switch (sel) {
+            case 3: NKLQ_Q2(true, true); break;
+            case 2: NKLQ_Q2(true, false); break;
+            case 1: NKLQ_Q2(false, true); break;
+            default: NKLQ_Q2(false, false); break;
+        }
+#undef NKLQ_Q2
     } else {
         const uint64_t items = m * n_cols;
         const uint32_t grid = grid_for_items(items);
         if (add)
-            hipLaunchKernelGGL((quant_2d_kernel<1, true>), dim3(grid), dim3(kBlock2D), 0, s, g, r_in,
+            hipLaunchKernelGGL((quant_2d_kernel<true>), dim3(grid), dim3(kBlock2D), 0, s, g, r_in,
                                r_out, c, n_rows, n_cols, items, thrd);
         else
-            hipLaunchKernelGGL((quant_2d_kernel<1, false>), dim3(grid), dim3(kBlock2D), 0, s, g, r_in,
+            hipLaunchKernelGGL((quant_2d_kernel<false>), dim3(grid), dim3(kBlock2D), 0, s, g, r_in,
                                r_out, c, n_rows, n_cols, items, thrd);
     }
     return launch_status();
@@ -827,12 +1091,18 @@ int nklq_dequantize_f32(float* out, const uint32_t* c, uint64_t n_rows, uint64_t
     }
     const uint64_t m = n_rows / 16 + (n_rows % 16 ? 1 : 0);
     if ((n_cols % 4 == 0) && aligned16(out) && aligned16(c)) {
-        const uint64_t items = m * (n_cols / 4);
-        hipLaunchKernelGGL((deq_2d_kernel<4>), dim3(grid_for_items(items)), dim3(kBlock2D), 0, s, out,
-                           c, n_rows, n_cols, items, thrd);
+        const uint64_t col_tiles = (n_cols + 255) / 256;
+        const uint64_t tiles = m * col_tiles;
+        if (tiles > 0x7FFFFFFFull || col_tiles > 0xFFFFFFFFull) return NKLQ_ERANGE;
+        if (g_nontemporal)
+            hipLaunchKernelGGL((deq_2d_rows_kernel<true>), dim3((uint32_t)tiles), dim3(kRowsBlock), 0, s,
+                               out, c, n_rows, n_cols, (uint32_t)col_tiles, thrd);
+        else
+            hipLaunchKernelGGL((deq_2d_rows_kernel<false>), dim3((uint32_t)tiles), dim3(kRowsBlock), 0,
+                               s, out, c, n_rows, n_cols, (uint32_t)col_tiles, thrd);
     } else {
         const uint64_t items = m * n_cols;
-        hipLaunchKernelGGL((deq_2d_kernel<1>), dim3(grid_for_items(items)), dim3(kBlock2D), 0, s, out,
+        hipLaunchKernelGGL((deq_2d_kernel), dim3(grid_for_items(items)), dim3(kBlock2D), 0, s, out,
                            c, n_rows, n_cols, items, thrd);
     }
     return launch_status();
@@ -861,6 +1131,112 @@ int nklq_dequant_accumulate_f32(float* acc, const uint32_t* const* payloads, int
         const int st = launch_acc_flat(acc, pl, k, n, thrd, acc_flag, s);
         if (st != NKLQ_OK) return st;
         acc_flag = 1;  // later launches continue the running sum held in acc
+    }
+    return NKLQ_OK;
+}
+
+int nklq_quantize_multi_f32(int count, const float* const* g, float* const* r, uint32_t* const* c,
+                            const uint64_t* n, float thrd, int add_residual, void* stream)
+{
+    if (count < 0) return NKLQ_ERANGE;
+    if (count == 0) return NKLQ_OK;
+    if (!g || !r || !c || !n) return NKLQ_ENULL;
+    for (int i = 0; i < count; ++i) {
+        if (n[i] == 0) continue;
+        if (!g[i] || !r[i] || !c[i]) return NKLQ_ENULL;
+        if (!aligned4(g[i]) || !aligned4(r[i]) || !aligned4(c[i])) return NKLQ_EALIGN;
+        if ((const void*)c[i] == (const void*)g[i] || (const void*)c[i] == (const void*)r[i])
+            return NKLQ_EALIAS;
+        if (n[i] / kChunk + 1 > 0x7FFFFFFFull) return NKLQ_ERANGE;
+    }
+    hipStream_t s = (hipStream_t)stream;
+    int i = 0;
+    while (i < count) {
+        QuantSegments seg = {};
+        bool al = true;
+        uint64_t chunks = 0;
+        int m = 0;
+        for (; i < count && m < kMaxSegments; ++i) {
+            if (n[i] == 0) continue;
+            const uint64_t mine = n[i] / kChunk + (n[i] % kChunk ? 1 : 0);
+            if (chunks + mine > 0x7FFFFFFFull) break;  // next launch
+            seg.g[m] = g[i];
+            seg.r[m] = r[i];
+            seg.c[m] = c[i];
+            seg.n[m] = n[i];
+            seg.first[m] = (uint32_t)chunks;
+            chunks += mine;
+            al = al && aligned16(g[i]) && aligned16(r[i]);
+            ++m;
+        }
+        seg.count = m;
+        for (int k = m; k <= kMaxSegments; ++k) seg.first[k] = (uint32_t)chunks;
+        if (m == 0) {
+            if (i < count) return NKLQ_ERANGE;  // a single vector that does not fit one launch
+            break;
+        }
+        const int st = launch_quant_multi(seg, al, add_residual != 0, thrd, s);
+        if (st != NKLQ_OK) return st;
+    }
+    return NKLQ_OK;
+}
+
+int nklq_dequant_accumulate_multi_f32(int count, float* const* acc, const uint64_t* n,
+                                      const uint64_t* word_offset,
+                                      const uint32_t* const* payload_base, int k_payloads,
+                                      float thrd, int accumulate, float divisor, void* stream)
+{
+    if (count < 0 || k_payloads < 1) return NKLQ_ERANGE;
+    if (count == 0) return NKLQ_OK;
+    if (!acc || !n || !word_offset || !payload_base) return NKLQ_ENULL;
+    for (int p = 0; p < k_payloads; ++p) {
+        if (!payload_base[p]) return NKLQ_ENULL;
+        if (!aligned4(payload_base[p])) return NKLQ_EALIGN;
+    }
+    for (int i = 0; i < count; ++i) {
+        if (n[i] == 0) continue;
+        if (!acc[i]) return NKLQ_ENULL;
+        if (!aligned4(acc[i])) return NKLQ_EALIGN;
+        if (n[i] / kTile + 1 > 0x7FFFFFFFull) return NKLQ_ERANGE;
+    }
+    hipStream_t s = (hipStream_t)stream;
+    int acc_flag = accumulate ? 1 : 0;
+    for (int first_p = 0; first_p < k_payloads; first_p += NKLQ_MAX_PAYLOADS_PER_LAUNCH) {
+        PayloadPtrs pl = {};
+        int k = k_payloads - first_p;
+        if (k > NKLQ_MAX_PAYLOADS_PER_LAUNCH) k = NKLQ_MAX_PAYLOADS_PER_LAUNCH;
+        for (int p = 0; p < k; ++p) pl.p[p] = payload_base[first_p + p];
+        for (int p = k; p < NKLQ_MAX_PAYLOADS_PER_LAUNCH; ++p) pl.p[p] = payload_base[first_p];
+        int i = 0;
+        while (i < count) {
+            AccSegments seg = {};
+            bool al = true;
+            uint64_t tiles = 0;
+            int m = 0;
+            for (; i < count && m < kMaxSegments; ++i) {
+                if (n[i] == 0) continue;
+                const uint64_t mine = n[i] / kTile + (n[i] % kTile ? 1 : 0);
+                if (tiles + mine > 0x7FFFFFFFull) break;
+                seg.acc[m] = acc[i];
+                seg.n[m] = n[i];
+                seg.word_offset[m] = word_offset[i];
+                seg.first[m] = (uint32_t)tiles;
+                tiles += mine;
+                al = al && aligned16(acc[i]);
+                ++m;
+            }
+            seg.count = m;
+            for (int j = m; j <= kMaxSegments; ++j) seg.first[j] = (uint32_t)tiles;
+            if (m == 0) {
+                if (i < count) return NKLQ_ERANGE;
+                break;
+            }
+            // the division belongs to the last group of payloads only
+            const bool last = first_p + NKLQ_MAX_PAYLOADS_PER_LAUNCH >= k_payloads;
+            const int st = launch_acc_multi(seg, pl, k, al, thrd, acc_flag, last ? divisor : 1.0f, s);
+            if (st != NKLQ_OK) return st;
+        }
+        acc_flag = 1;
     }
     return NKLQ_OK;
 }

@@ -212,3 +212,88 @@ def cu_fn_dequantize_accumulate_e(acc, payloads, thrd=0.3, accumulate=False, str
         _lib.check(_lib.lib().nklq_dequant_accumulate_f32(
             acc.data_ptr(), ptrs, len(payloads), n, float(thrd), 1 if accumulate else 0, h))
         _finish(stream, acc.device, sync)
+
+
+# ------------------------------------------------------------------ many vectors per launch
+
+def _ptr_array(ptrs):
+    return (ct.c_void_p * len(ptrs))(*ptrs)
+
+
+def cu_fn_quantize_multi_e(grads, comps, resis, thrd=0.3, add_residual=True, stream=None, sync=True):
+    """Flat quantize of many vectors with one launch per 32 of them.
+
+    ``grads[i]``, ``resis[i]``: float32 GPU tensors of the same number of elements (any shape,
+    contiguous); ``comps[i]``: ceil(numel/16) words.  With ``add_residual`` the residual is read,
+    added to the gradient and updated in place (error feedback); otherwise it is only written.
+    The per-parameter form of necklace's buffers (grd_resi / grd_comp lists,
+    necklace/trainer/tnopmx.py:140-149) maps onto this directly.
+    """
+    if not (len(grads) == len(comps) == len(resis)):
+        raise ValueError("grads, comps and resis must have the same length")
+    if not grads:
+        return
+    dev = grads[0].device
+    ns = []
+    for i, (gr, cm, rs) in enumerate(zip(grads, comps, resis)):
+        _check_f32(f"grads[{i}]", gr.reshape(-1) if isinstance(gr, torch.Tensor) and gr.dim() > 2 else gr)
+        _check_f32(f"resis[{i}]", rs.reshape(-1) if isinstance(rs, torch.Tensor) and rs.dim() > 2 else rs)
+        n = gr.numel()
+        if rs.numel() != n:
+            raise ValueError(f"resis[{i}] has {rs.numel()} elements, grads[{i}] has {n}")
+        _check_words(f"comps[{i}]", cm, n, 1, 1)
+        if not (gr.device == cm.device == rs.device == dev):
+            raise ValueError("all tensors must be on the same GPU")
+        ns.append(n)
+    with torch.cuda.device(dev):
+        h = nbutils.stream_handle(stream, dev)
+        _lib.check(_lib.lib().nklq_quantize_multi_f32(
+            len(ns), _ptr_array([t.data_ptr() for t in grads]), _ptr_array([t.data_ptr() for t in resis]),
+            _ptr_array([t.data_ptr() for t in comps]), (ct.c_uint64 * len(ns))(*ns), float(thrd),
+            1 if add_residual else 0, h))
+        _finish(stream, dev, sync)
+
+
+def cu_fn_dequantize_accumulate_multi_e(accs, word_offsets, payloads, thrd=0.3, accumulate=False,
+                                        divisor=1.0, stream=None, sync=True):
+    """Fixed-order decode-and-sum into many vectors with one launch per 32 of them.
+
+    ``payloads``: one 2-D tensor [K, W] (or a list of K 1-D tensors of W words): the message of
+    each of the K peers.  Vector i (``accs[i]``, float32, contiguous) has its code words at
+    ``word_offsets[i]`` in every message.  Same sum as `cu_fn_dequantize_accumulate_e`; the
+    result is divided by `divisor` (true division) when it is not 1.
+    """
+    if len(accs) != len(word_offsets):
+        raise ValueError("accs and word_offsets must have the same length")
+    if isinstance(payloads, torch.Tensor):
+        if payloads.dim() != 2:
+            raise TypeError("payloads: expected a sequence of 1-D tensors or one 2-D tensor")
+        payloads = list(payloads.unbind(0))
+    if len(payloads) < 1:
+        raise ValueError("payloads: at least one is required")
+    if not accs:
+        return
+    dev = accs[0].device
+    w_total = payloads[0].numel()
+    for i, p in enumerate(payloads):
+        if not isinstance(p, torch.Tensor) or p.dtype not in _WORD_DTYPES or p.dim() != 1:
+            raise TypeError(f"payloads[{i}]: expected a 1-D uint32/int32 tensor")
+        if not p.is_cuda or not p.is_contiguous() or p.numel() != w_total or p.device != dev:
+            raise ValueError(f"payloads[{i}]: must be contiguous, on the same GPU and of equal length")
+    ns = []
+    for i, (a, wo) in enumerate(zip(accs, word_offsets)):
+        _check_f32(f"accs[{i}]", a.reshape(-1) if isinstance(a, torch.Tensor) and a.dim() > 2 else a)
+        if a.device != dev:
+            raise ValueError("all tensors must be on the same GPU")
+        n = a.numel()
+        if wo < 0 or wo + packed_rows(n) > w_total:
+            raise ValueError(f"vector {i}: words [{wo}, {wo + packed_rows(n)}) exceed the payload length {w_total}")
+        ns.append(n)
+    with torch.cuda.device(dev):
+        h = nbutils.stream_handle(stream, dev)
+        _lib.check(_lib.lib().nklq_dequant_accumulate_multi_f32(
+            len(ns), _ptr_array([t.data_ptr() for t in accs]), (ct.c_uint64 * len(ns))(*ns),
+            (ct.c_uint64 * len(ns))(*[int(w) for w in word_offsets]),
+            _ptr_array([p.data_ptr() for p in payloads]), len(payloads), float(thrd),
+            1 if accumulate else 0, float(divisor), h))
+        _finish(stream, dev, sync)

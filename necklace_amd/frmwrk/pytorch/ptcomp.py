@@ -26,8 +26,12 @@ Semantics that the reference leaves open and this module fixes: error feedback
 is an fp32 add before quantizing; the sum over ranks is a strict left-to-right
 fp32 sum in rank order (fp32 sums of {0, +t, -t} depend on the order).
 """
+import ctypes as ct
+
 import torch
 
+from ... import _lib
+from ...cuda import nbutils as _nb
 from ...cuda import quantize as _q
 
 CMP_RATIO = _q.CMP_RATIO
@@ -113,6 +117,35 @@ class GradCompressor:
                 self.grd_resi.append(None)
                 self.grd_comp.append(None)
                 self.grd_recv.append(None)
+        # argument tables of the many-vectors entry points; everything but the gradients' own
+        # addresses is fixed for the life of the buffers
+        self._idx = [i for i, c in enumerate(self.grd_cmps) if c]
+        m = len(self._idx)
+        self._n_arr = (ct.c_uint64 * m)(*[lay.numels[i] for i in self._idx])
+        self._wo_arr = (ct.c_uint64 * m)(*[lay.word_offset[i] for i in self._idx])
+        self._r_arr = (ct.c_void_p * m)(*[self.grd_resi[i].data_ptr() for i in self._idx])
+        self._c_arr = (ct.c_void_p * m)(*[self.grd_comp[i].data_ptr() for i in self._idx])
+        self._pl_arr = (ct.c_void_p * self.kn)(*[self.recv[k].data_ptr() for k in range(self.kn)])
+
+    def _ptrs(self, tensors, what):
+        """Device addresses of the compressed parameters' tensors, after checking them."""
+        if len(tensors) != len(self.layout):
+            raise ValueError(f"expected {len(self.layout)} {what}s, got {len(tensors)}")
+        for i in self._idx:
+            if tensors[i].numel() != self.layout.numels[i]:
+                raise ValueError(
+                    f"{what} {i}: {tensors[i].numel()} elements, layout has {self.layout.numels[i]}")
+        out = []
+        for i in self._idx:
+            t = tensors[i]
+            if t.dtype != torch.float32 or not t.is_cuda:
+                raise TypeError(f"{what} {i}: expected a float32 GPU tensor, got {t.dtype} on {t.device}")
+            if not t.is_contiguous():
+                raise ValueError(f"{what} {i} must be contiguous")
+            if t.device != self.resi.device:
+                raise ValueError(f"{what} {i} is on {t.device}, the buffers are on {self.resi.device}")
+            out.append(t.data_ptr())
+        return (ct.c_void_p * len(out))(*out)
 
     # ---- send side
 
@@ -120,18 +153,15 @@ class GradCompressor:
         """Quantize every compressed parameter's gradient with error feedback.
 
         `grads[i]` is parameter i's gradient (any shape, contiguous fp32 on the GPU);
-        entries of uncompressed parameters are ignored.  One launch per parameter.
+        entries of uncompressed parameters are ignored.  One launch per 32 parameters.
         """
-        if len(grads) != len(self.layout):
-            raise ValueError(f"expected {len(self.layout)} gradients, got {len(grads)}")
-        for i, g in enumerate(grads):
-            if self.grd_cmps[i] and g.numel() != self.layout.numels[i]:
-                raise ValueError(f"gradient {i}: {g.numel()} elements, layout has {self.layout.numels[i]}")
-        for i, g in enumerate(grads):
-            if not self.grd_cmps[i]:
-                continue
-            _q.cu_fn_matrix_quantize_e(g.reshape(-1), self.grd_comp[i], self.grd_resi[i], self.thrd,
-                                       stream=stream, add_residual=True, sync=False)
+        g_arr = self._ptrs(grads, "gradient")
+        if not self._idx:
+            return
+        with torch.cuda.device(self.resi.device):
+            _lib.check(_lib.lib().nklq_quantize_multi_f32(
+                len(self._idx), g_arr, self._r_arr, self._c_arr, self._n_arr, self.thrd, 1,
+                _nb.stream_handle(stream, self.resi.device)))
         if sync:
             _sync(self.device, stream)
 
@@ -155,22 +185,13 @@ class GradCompressor:
     def decompress_sum(self, outs, average=True, stream=None, sync=False):
         """outs[i] <- sum over ranks k = 0..kn-1 (in that order) of decode(recv[k] of parameter i),
         divided by kn when `average` (the `/ kn` of necklace/frmwrk/pytorch/ptprms.py:294)."""
-        if len(outs) != len(self.layout):
-            raise ValueError(f"expected {len(self.layout)} outputs, got {len(outs)}")
-        for i, o in enumerate(outs):
-            if not self.grd_cmps[i]:
-                continue
-            if not o.is_contiguous() or o.numel() != self.layout.numels[i]:
-                raise ValueError(f"output {i} must be contiguous with {self.layout.numels[i]} elements")
-            flat = o.view(-1)
-            _q.cu_fn_dequantize_accumulate_e(flat, self.grd_recv[i], self.thrd, accumulate=False,
-                                             stream=stream, sync=False)
-            if average and self.kn > 1:
-                if stream is None:
-                    flat.div_(self.kn)
-                else:
-                    with torch.cuda.stream(stream):
-                        flat.div_(self.kn)
+        o_arr = self._ptrs(outs, "output")
+        if not self._idx:
+            return
+        with torch.cuda.device(self.resi.device):
+            _lib.check(_lib.lib().nklq_dequant_accumulate_multi_f32(
+                len(self._idx), o_arr, self._n_arr, self._wo_arr, self._pl_arr, self.kn, self.thrd, 0,
+                float(self.kn) if average else 1.0, _nb.stream_handle(stream, self.resi.device)))
         if sync:
             _sync(self.device, stream)
 

@@ -226,3 +226,60 @@ def test_round_trip_and_zero_residual_on_gpu():
     C2, R2 = gpu_quantize(d, 2e-3)
     assert_words_equal(C2, C)
     assert not R2.any()
+
+
+def test_many_vectors_in_one_launch(knobs):
+    """nklq_quantize_multi_f32 / nklq_dequant_accumulate_multi_f32: 45 vectors of awkward lengths
+    (more than one table of 32), some at odd element offsets, each equal to its own flat result."""
+    sizes = [1, 15, 16, 17, 255, 256, 257, 511, 1023, 1024, 1025, 2047, 4096, 5000, 70001] * 3
+    rng = np.random.default_rng(314)
+    thrd, K = 1e-3, 3
+    arena_g = torch.zeros(sum(sizes) + 4 * len(sizes), device="cuda")
+    arena_r = torch.zeros_like(arena_g)
+    grads, resis, comps, gh, rh = [], [], [], [], []
+    pos = 0
+    for i, n in enumerate(sizes):
+        off = pos + (i % 4)  # every alignment class of the base address
+        g = rng.normal(0, 1e-3, n).astype(np.float32)
+        r = rng.normal(0, 5e-4, n).astype(np.float32)
+        arena_g[off:off + n].copy_(torch.from_numpy(g))
+        arena_r[off:off + n].copy_(torch.from_numpy(r))
+        grads.append(arena_g[off:off + n])
+        resis.append(arena_r[off:off + n])
+        comps.append(words_like(n))
+        gh.append(g)
+        rh.append(r)
+        pos += n + 4
+    q.cu_fn_quantize_multi_e(grads, comps, resis, thrd, add_residual=True)
+    for i, n in enumerate(sizes):
+        want_c, want_r = oracle.c.quantize(gh[i], thrd, R_in=rh[i])
+        assert_words_equal(host_words(comps[i]), want_c, f"vector {i} n={n}")
+        assert_bits_equal(resis[i].cpu().numpy(), want_r, f"vector {i} n={n}")
+    # plain form: residual only written
+    outs = [torch.full((n,), 3.0, device="cuda") for n in sizes]
+    q.cu_fn_quantize_multi_e(grads, comps, outs, thrd, add_residual=False)
+    for i in (0, 4, 9, 14, 44):
+        want_c, want_r = oracle.c.quantize(gh[i], thrd)
+        assert_words_equal(host_words(comps[i]), want_c)
+        assert_bits_equal(outs[i].cpu().numpy(), want_r)
+    # receive side: K messages, vector i's words at word_offsets[i] in each
+    woffs, w = [], 0
+    for n in sizes:
+        woffs.append(w)
+        w += (n + 15) // 16 + 1  # a gap word between vectors
+    msgs = rng.integers(0, 2 ** 32, size=(K, w), dtype=np.uint64).astype(np.uint32)
+    dmsgs = dev(msgs)
+    for acc0 in (False, True):
+        accs = [torch.full((n,), 0.5, device="cuda") for n in sizes]
+        q.cu_fn_dequantize_accumulate_multi_e(accs, woffs, dmsgs, thrd, accumulate=acc0)
+        for i, n in enumerate(sizes):
+            pl = [msgs[k, woffs[i]:woffs[i] + (n + 15) // 16].copy() for k in range(K)]
+            want = oracle.c.dequant_accumulate(pl, n, thrd, acc=np.full(n, 0.5, np.float32) if acc0 else None)
+            assert_bits_equal(accs[i].cpu().numpy(), want, f"vector {i} n={n} accumulate={acc0}")
+    # with the division by the number of workers folded in (7 is not a power of two)
+    accs = [torch.empty(n, device="cuda") for n in sizes]
+    q.cu_fn_dequantize_accumulate_multi_e(accs, woffs, dmsgs, thrd, divisor=7.0)
+    for i, n in enumerate(sizes):
+        pl = [msgs[k, woffs[i]:woffs[i] + (n + 15) // 16].copy() for k in range(K)]
+        want = (oracle.c.dequant_accumulate(pl, n, thrd) / np.float32(7.0)).astype(np.float32)
+        assert_bits_equal(accs[i].cpu().numpy(), want, f"vector {i} n={n} divided")
