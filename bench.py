@@ -41,7 +41,10 @@ def parse():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--elems", type=int, default=N_ELEMS, help="gradient length (default: the headline size)")
-    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU-baseline time budget; 0 skips it")
+    ap.add_argument("--chunk", type=int, default=0,
+                    help="elements per launch (multiple of 16); 0 = the whole gradient in one launch. "
+                         "The HBM-sizing workload is --elems 2800000000 --chunk 268435456")
+    ap.add_argument("--cpu-seconds", type=float, default=20.0, help="CPU-baseline time budget; 0 skips it")
     ap.add_argument("--legs", default="deq,acc,copy,cpu",
                     help="extra legs after the timed quantize steps: deq, acc, copy, cpu (comma list, '' = none)")
     return ap.parse_args()
@@ -75,22 +78,32 @@ def time_region(torch, fn, steps):
     return wall_ms, e0.elapsed_time(e1)
 
 
+def _time_passes(fn, budget_s, max_reps=10000):
+    fn()  # warm: page in, spin up threads
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        fn()
+        reps += 1
+        el = time.perf_counter() - t0
+        if el >= budget_s or reps >= max_reps:
+            return reps, el
+
+
 def cpu_baseline(g_slab, r_slab, budget_s):
-    """Time the CPU restatement of the reference kernel on a slab of the workload."""
+    """Time the CPU restatement of the reference kernel on a slab of the workload: the C version on
+    all host threads (the headline baseline), on one thread, and the numpy version."""
     import numpy as np
     import oracle
     threads = oracle.c.threads()
     n = g_slab.shape[0]
     c = np.empty((n + 15) // 16, dtype=np.uint32)
     r = r_slab.copy()
-    oracle.c.fused_quantize_inplace(g_slab, r, c, THRD)  # warm: page in, spin up threads
-    reps, t0 = 0, time.perf_counter()
-    while True:
-        oracle.c.fused_quantize_inplace(g_slab, r, c, THRD)
-        reps += 1
-        el = time.perf_counter() - t0
-        if el >= budget_s or reps >= 10000:
-            break
+    reps, el = _time_passes(lambda: oracle.c.fused_quantize_inplace(g_slab, r, c, THRD), budget_s * 0.6)
+    oracle.c.set_threads(1)
+    reps1, el1 = _time_passes(lambda: oracle.c.fused_quantize_inplace(g_slab, r, c, THRD), budget_s * 0.2)
+    oracle.c.set_threads(threads)
+    m = min(n, 1 << 22)
+    repsn, eln = _time_passes(lambda: oracle.vec.quantize(g_slab[:m], THRD, R_in=r_slab[:m]), budget_s * 0.2)
     return {
         "value": round(BYTES_QUANT * n * reps / el / 1e9, 3),
         "unit": "GB/s",
@@ -99,6 +112,8 @@ def cpu_baseline(g_slab, r_slab, budget_s):
         "elements_per_s": round(n * reps / el),
         "sample": f"{reps} passes over the first {n} elements of the same gradient "
                   f"({el:.1f} s, C restatement of necklace/cuda/quantize.py, OpenMP {threads} threads)",
+        "one_thread_GBps": round(BYTES_QUANT * n * reps1 / el1 / 1e9, 3),
+        "numpy_one_thread_GBps": round(BYTES_QUANT * m * repsn / eln / 1e9, 3),
     }
 
 
@@ -127,17 +142,25 @@ def main():
     c = torch.empty(_lib.packed_words(n), dtype=torch.int32, device="cuda")
     stream = torch.cuda.current_stream().cuda_stream
 
+    if args.chunk < 0 or args.chunk % 16:
+        print("bench.py: --chunk must be a non-negative multiple of 16", file=sys.stderr)
+        sys.exit(2)
+    chunk = args.chunk or n
+    pieces = [(lo, min(n, lo + chunk)) for lo in range(0, n, chunk)]
+    gp, rp, cp = g.data_ptr(), r.data_ptr(), c.data_ptr()
+
     def step():
-        _lib.check(L.nklq_quantize_f32(g.data_ptr(), r.data_ptr(), r.data_ptr(), c.data_ptr(),
-                                       n, 1, THRD, 1, stream))
+        for lo, hi in pieces:
+            _lib.check(L.nklq_quantize_f32(gp + 4 * lo, rp + 4 * lo, rp + 4 * lo, cp + 4 * (lo // 16),
+                                           hi - lo, 1, THRD, 1, stream))
 
     for _ in range(args.warmup):
         step()
     wall_ms, ev_ms = time_region(torch, step, args.steps)
     ms_per_step = wall_ms / args.steps
-    kernel_ms = ev_ms / args.steps
-    bytes_per_launch = BYTES_QUANT * n
-    value = bytes_per_launch / (ms_per_step * 1e-3) / 1e9
+    kernel_ms = ev_ms / args.steps / len(pieces)
+    bytes_per_launch = BYTES_QUANT * n / len(pieces)
+    value = BYTES_QUANT * n / (ms_per_step * 1e-3) / 1e9
     achieved = bytes_per_launch / (kernel_ms * 1e-3) / 1e9
 
     traffic = None
@@ -149,7 +172,8 @@ def main():
             traffic = None
 
     res = {
-        "metric": "fused 2-bit quantize GB/s (355M fp32 grad)",
+        "metric": "fused 2-bit quantize GB/s (355M fp32 grad)" if n == N_ELEMS
+                  else f"fused 2-bit quantize GB/s ({n}-element fp32 grad)",
         "value": round(value, 1),
         "unit": "GB/s",
         "n_gpus": 1,
@@ -162,12 +186,14 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {
-            "workload": "GPT-2-medium-sized flat fp32 gradient, fused quantize + residual update + pack",
+            "workload": ("GPT-2-medium-sized" if n == N_ELEMS else f"{n}-element")
+                        + " flat fp32 gradient, fused quantize + residual update + pack",
             "elements": n,
             "gradient": "1e-3 * Student-t(df=3), generated on the GPU",
             "residual": "N(0, sigma=1e-4) at step 0, carried in place across steps",
             "thrd": THRD,
             "layout": "flat (N,1): word w packs elements 16w..16w+15",
+            "launches_per_step": len(pieces),
         },
         "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
         "roofline": {
