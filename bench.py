@@ -46,7 +46,8 @@ def parse():
                          "The HBM-sizing workload is --elems 2800000000 --chunk 268435456")
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="CPU-baseline time budget; 0 skips it")
     ap.add_argument("--legs", default="deq,acc,copy,cpu",
-                    help="extra legs after the timed quantize steps: deq, acc, copy, cpu (comma list, '' = none)")
+                    help="extra legs after the timed quantize steps: deq, acc, copy, cpu, and (off by "
+                         "default) matrix, multi (comma list, '' = none)")
     return ap.parse_args()
 
 
@@ -256,6 +257,61 @@ def main():
             "elements_per_s": round(nb / (acc_ms * 1e-3)),
             "ms": round(acc_ms, 4),
             "GBps": round(acc_bytes / (acc_ms * 1e-3) / 1e9, 1),
+        }
+
+    if "matrix" in legs:
+        # the reference's own layout: (n, k) matrix, codes packed down the columns
+        side = 8192
+        A = g[:side * side].view(side, side)
+        R = torch.zeros(side, side, device="cuda")
+        C = torch.empty(side // 16, side, dtype=torch.int32, device="cuda")
+
+        def mq():
+            _lib.check(L.nklq_quantize_f32(A.data_ptr(), R.data_ptr(), R.data_ptr(), C.data_ptr(),
+                                           side, side, THRD, 1, stream))
+
+        def md():
+            _lib.check(L.nklq_dequantize_f32(R.data_ptr(), C.data_ptr(), side, side, THRD, stream))
+
+        for _ in range(5):
+            mq()
+        _, ev = time_region(torch, mq, 50)
+        res["matrix_8192x8192"] = {"fused_GBps": round(BYTES_QUANT * side * side / (ev / 50 * 1e-3) / 1e9, 1)}
+        for _ in range(5):
+            md()
+        _, ev = time_region(torch, md, 50)
+        res["matrix_8192x8192"]["decode_GBps"] = round(BYTES_DEQUANT * side * side / (ev / 50 * 1e-3) / 1e9, 1)
+        del A, R, C
+
+    if "multi" in legs:
+        # a ResNet-50-shaped list of gradient tensors through the trainer-side buffers
+        from necklace_amd.frmwrk.pytorch import ptcomp
+        sizes = [64 * 3 * 7 * 7, 64, 64]
+        inpl = 64
+        for planes, blocks in ((64, 3), (128, 4), (256, 6), (512, 3)):
+            for b in range(blocks):
+                sizes += [planes * inpl, planes, planes, planes * planes * 9, planes, planes,
+                          4 * planes * planes, 4 * planes, 4 * planes]
+                if b == 0:
+                    sizes += [4 * planes * inpl, 4 * planes, 4 * planes]
+                inpl = 4 * planes
+        sizes += [1000 * 2048, 1000]
+        gcomp = ptcomp.GradCompressor(sizes, K_PAYLOADS, thrd=THRD)
+        gl, pos = [], 0
+        for sz in sizes:
+            gl.append(g[pos:pos + sz])
+            pos += sz
+        gcomp.recv.random_(-2 ** 31, 2 ** 31 - 1)
+        outs = [torch.empty(sz, device="cuda") for sz in sizes]
+        nel = sum(sz for sz in sizes if sz >= 1001)
+        for _ in range(5):
+            gcomp.compress(gl)
+            gcomp.decompress_sum(outs)
+        _, ev = time_region(torch, lambda: gcomp.compress(gl), 50)
+        _, ev2 = time_region(torch, lambda: gcomp.decompress_sum(outs), 50)
+        res["resnet50_tensor_list"] = {
+            "tensors": len(sizes), "compressed_elements": nel,
+            "compress_us": round(ev / 50 * 1e3, 1), "decompress_sum_us": round(ev2 / 50 * 1e3, 1),
         }
 
     if "copy" in legs:
