@@ -272,3 +272,52 @@ def grads_do_compressed_exchange(grads, kn, grad_comp_cfg, exchange=None, averag
         raise ValueError("an exchange callable is required when kn > 1")
     gc.decompress_sum(grads, average=average, stream=stream)
     return [i for i, c in enumerate(gc.grd_cmps) if not c]
+
+
+# --------------------------------------------------------------------------- flat gradient buffer
+
+def init_flat_grad_comp_cfg(total_size, kn, grad_comp_cfg=None, device="cuda", rank=0):
+    """`grad_comp_cfg` for ONE flat gradient buffer of `total_size` floats — the `grd_fltn_gpu` of
+    PtCudaFltnMemManager (necklace/frmwrk/pytorch/tsmem.py:157-180), which the flat ZeRO trainer
+    reduces as a whole (necklace/trainer/zroppf.py:957-965).  Residual, payload and receive slots
+    are allocated once, next to it; the buffer itself is never copied."""
+    cfg = dict(grad_comp_cfg or {})
+    cfg["grad_size_threshold"] = 1  # a flat buffer is always compressed
+    return init_grad_comp_cfg([int(total_size)], kn, cfg, device=device, rank=rank)
+
+
+def opt_grads_fltn_do_compressed_reduce(kn, d_arr_send, sz, grad_comp_cfg, exchange=None, average=False,
+                                        stream=None):
+    """Compressed form of ``opt_grads_fltn_do_nccl_reduce(nc, kn, root, d_arr_send, sz, grad_comp_cfg)``
+    (necklace/frmwrk/pytorch/ptprms.py:396-401): the first `sz` floats of the flat buffer
+    `d_arr_send` are quantized with error feedback (one launch per 2^28 elements), `exchange(comp,
+    recv)` gathers every rank's payload, and the decoded sum over ranks, in rank order, replaces
+    them.  The reference's reduce does not average; pass ``average=True`` for ``/ kn``."""
+    gc = grad_comp_cfg["compressor"]
+    if gc.kn != kn:
+        raise ValueError(f"grad_comp_cfg was built for kn={gc.kn}, got kn={kn}")
+    flat = d_arr_send.reshape(-1)[:sz]
+    gc.compress_flat(flat, stream=stream)
+    if exchange is not None:
+        exchange(gc.comp, gc.recv)
+    elif kn != 1:
+        raise ValueError("an exchange callable is required when kn > 1")
+    gc.decompress_sum([flat], average=average, stream=stream)
+
+
+# --------------------------------------------------------------------------- checkpoint
+
+def grad_comp_state(grad_comp_cfg):
+    """What has to go into the `state` dict handed to save_checkpoint
+    (necklace/frmwrk/pytorch/callback.py:16-19) for the error feedback to survive a restart:
+    the residual and the layout it belongs to.  Plain tensors and numbers only, so the file
+    loads with ``torch.load(..., weights_only=True)``."""
+    st = grad_comp_cfg["compressor"].state_dict()
+    return {"resi": st["resi"].detach().clone(), "thrd": float(st["thrd"]),
+            "numels": [int(n) for n in st["numels"]], "size_threshold": int(st["size_threshold"])}
+
+
+def load_grad_comp_state(grad_comp_cfg, state):
+    """Restore what `grad_comp_state` saved into a `grad_comp_cfg` built for the same parameters."""
+    grad_comp_cfg["compressor"].load_state_dict(state)
+    grad_comp_cfg["grad_comp_threshold"] = float(state["thrd"])

@@ -92,3 +92,50 @@ def test_residual_state_survives_a_restart():
     torch.cuda.synchronize()
     assert torch.equal(a.resi.view(torch.int32), b.resi.view(torch.int32))
     assert torch.equal(a.comp, b.comp)
+
+
+def test_flat_zero_style_buffer_reduce_in_place():
+    """One flat gradient buffer (the grd_fltn_gpu of the flat ZeRO trainer): compress in place,
+    two synthetic peers, decoded sum written back over the gradient; nothing is copied."""
+    total, kn, rank, thrd = 1_500_000 + 9, 3, 2, 2e-3
+    cfg = ptcomp.init_flat_grad_comp_cfg(total, kn, {"grad_comp_threshold": thrd}, rank=rank)
+    gc = cfg["compressor"]
+    rng = np.random.default_rng(31)
+    resid = np.zeros(total, np.float32)
+    for step in range(2):
+        g = rng.normal(0, 2e-3, total).astype(np.float32)
+        buf = dev(g)
+        peers = random_payloads_gpu(kn, 16 * gc.layout.total_words, 40 + step)
+
+        def exchange(comp, recv, peers=peers):
+            mine = comp.clone()
+            recv.copy_(peers)
+            recv[rank].copy_(mine)
+
+        ptr = buf.data_ptr()
+        ptcomp.opt_grads_fltn_do_compressed_reduce(kn, buf, total, cfg, exchange=exchange)
+        torch.cuda.synchronize()
+        assert buf.data_ptr() == ptr
+        want_c, resid = oracle.c.quantize(g, thrd, R_in=resid)
+        ph = host_words(peers)
+        w = gc.layout.words[0]
+        pl = [ph[k, :w].copy() for k in range(kn)]
+        pl[rank] = want_c
+        assert_words_equal(host_words(gc.grd_comp[0]), want_c, f"step {step}")
+        assert_bits_equal(gc.grd_resi[0].cpu().numpy(), resid, f"step {step}")
+        assert_bits_equal(buf.cpu().numpy(), oracle.c.dequant_accumulate(pl, total, thrd), f"step {step}")
+
+
+def test_checkpoint_file_round_trip(tmp_path):
+    n, thrd = 20_000, 1e-3
+    cfg = ptcomp.init_flat_grad_comp_cfg(n, 1, {"grad_comp_threshold": thrd})
+    g = dev(np.random.default_rng(2).normal(0, 1e-3, n).astype(np.float32))
+    cfg["compressor"].compress_flat(g, sync=True)
+    path = tmp_path / "checkpoint.pth.tar"
+    torch.save({"epoch": 3, "grad_comp": ptcomp.grad_comp_state(cfg)}, path)
+    state = torch.load(path, weights_only=True)
+    cfg2 = ptcomp.init_flat_grad_comp_cfg(n, 1, {"grad_comp_threshold": 0.5})
+    ptcomp.load_grad_comp_state(cfg2, state["grad_comp"])
+    assert cfg2["compressor"].thrd == thrd
+    assert torch.equal(cfg2["compressor"].resi.view(torch.int32), cfg["compressor"].resi.view(torch.int32))
+    assert state["epoch"] == 3
