@@ -126,6 +126,8 @@ def main():
         sys.exit(2)
 
     import torch
+    from necklace_amd.csrc import build as hip_build
+    hip_build.ensure_built()  # compiles only when no library is there; a failed build raises
     from necklace_amd import _lib
     from necklace_amd.cuda import quantize as q  # noqa: F401  (fails loudly if the library is missing)
 

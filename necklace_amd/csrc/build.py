@@ -41,5 +41,12 @@ def build(verbose=False):
     return SO_PATH
 
 
+def ensure_built():
+    """Build only when no library is there yet (a fresh checkout: the .so is not in version control)."""
+    if not os.path.exists(SO_PATH):
+        build()
+    return SO_PATH
+
+
 if __name__ == "__main__":
     print(build(verbose="-q" not in sys.argv))

@@ -12,6 +12,11 @@ if ROOT not in sys.path:
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+    # a fresh checkout has no built libraries (they are not in version control): build them once
+    from necklace_amd.csrc import build as hip_build
+    hip_build.ensure_built()
+    import oracle
+    oracle.c.lib()
 
 
 def bits_to_f32(hexes):
