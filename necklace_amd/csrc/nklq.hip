@@ -38,11 +38,11 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 // flat buffer (torch.narrow) start at any element.  gfx950 global memory
 // instructions need dword alignment only, so these still move 16 bytes per lane.
 typedef f32x4 f32x4_a4 __attribute__((aligned(4)));
+typedef u32x4 u32x4_a4 __attribute__((aligned(4)));
 
 constexpr int kWave = 64;
 constexpr int kChunk = 256;          // elements per chunk: one dwordx4 per lane
 constexpr int kWordsPerChunk = 16;
-constexpr int kBlock2D = 256;        // workgroup size of the general matrix kernels
 
 // ---------------------------------------------------------------- per element
 
@@ -373,10 +373,123 @@ __global__ __launch_bounds__(BLOCK) void acc_flat_kernel(
 
 // ---------------------------------------------------------------- matrix (n, k) kernels
 
-// Word (x, y) packs rows 16x .. 16x+15 of column y (quantize.py:35-51).
-//
-// General form, any k and any 4-byte-aligned bases: one lane per word, lanes walk along y (the
-// contiguous dimension), so a wave reads 256 B of each of its 16 rows.
+// Word (x, y) packs rows 16x .. 16x+15 of column y (quantize.py:35-51), so the 16 codes of a
+// word are k floats apart in memory.  A workgroup of 16 waves takes a tile of 16 rows x 256
+// columns: wave i moves row 16x+i of the tile with one dwordx4 per lane (1 KiB contiguous, like
+// a flat chunk), so neighbouring workgroups (on different XCDs) touch neighbouring 1 KiB pieces
+// of the same rows.  The 16 codes of a word come from 16 different waves: each wave ORs its
+// code, shifted to its bit position, into the tile's 256 words in LDS; after a barrier 256
+// threads store the 1 KiB of words.  When k is not a multiple of 4 (or a base is not 16-byte
+// aligned) rows start at any element: ALIGNED = false issues the same loads with dword
+// alignment, and the last 1-3 columns of a row are moved one by one.
+constexpr int kRowsBlock = 16 * kWave;  // 1024 threads
+constexpr uint64_t kNarrowColumns = 64; // below this many columns the one-lane-per-word kernels run
+
+template <bool ADD, bool NT, bool ALIGNED>
+__global__ __launch_bounds__(kRowsBlock) void quant_2d_rows_kernel(
+    const float* g, const float* rin, float* rout, uint32_t* __restrict__ c, uint64_t n,
+    uint64_t k, uint32_t col_tiles, float t)
+{
+    __shared__ uint32_t words[256];
+    const int lane = threadIdx.x & (kWave - 1);
+    const uint32_t i = threadIdx.x >> 6;  // row inside the tile = code position inside the word
+    const uint64_t x = blockIdx.x / col_tiles;
+    const uint64_t y0 = (uint64_t)(blockIdx.x % col_tiles) * 256;
+    const uint64_t y = y0 + (uint64_t)lane * 4;
+    const uint64_t row = x * 16 + i;
+    // columns this lane owns: 4, or fewer at the right edge, or none
+    // (with ALIGNED, k is a multiple of 4: it is 4 or none)
+    const int cnt = (row < n && y < k) ? ((ALIGNED || k - y >= 4) ? 4 : (int)(k - y)) : 0;
+    const uint64_t off = row * k + y;
+    float a[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    float r[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (cnt == 4) {
+        const f32x4 va = ld4<ALIGNED, NT>(g + off);
+        a[0] = va.x; a[1] = va.y; a[2] = va.z; a[3] = va.w;
+        if constexpr (ADD) {
+            const f32x4 vr = ld4<ALIGNED, NT>(rin + off);
+            r[0] = vr.x; r[1] = vr.y; r[2] = vr.z; r[3] = vr.w;
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < 3; ++j) {
+            if (j < cnt) {
+                a[j] = g[off + j];
+                if constexpr (ADD) r[j] = rin[off + j];
+            }
+        }
+    }
+    if (threadIdx.x < 256) words[threadIdx.x] = 0;
+    __syncthreads();
+    if (cnt > 0) {
+        float o[4];
+        uint32_t code[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            float v = a[j];
+            if constexpr (ADD) v = v + r[j];
+            code[j] = quant_one(v, t, o[j]);
+        }
+        if (cnt == 4) {
+            f32x4 vo;
+            vo.x = o[0]; vo.y = o[1]; vo.z = o[2]; vo.w = o[3];
+            st4<ALIGNED, NT>(rout + off, vo);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 3; ++j)
+                if (j < cnt) rout[off + j] = o[j];
+        }
+        const uint32_t sh = 2 * i;
+        // column 4*lane + j lives at words[64*j + lane]: consecutive lanes, consecutive banks
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (j < cnt && code[j]) atomicOr(&words[64 * j + lane], code[j] << sh);
+    }
+    __syncthreads();
+    if (threadIdx.x < 256 && y0 + threadIdx.x < k)
+        c[x * k + y0 + threadIdx.x] = words[64 * (threadIdx.x & 3) + (threadIdx.x >> 2)];
+}
+
+template <bool NT, bool ALIGNED>
+__global__ __launch_bounds__(kRowsBlock) void deq_2d_rows_kernel(
+    float* out, const uint32_t* __restrict__ c, uint64_t n, uint64_t k, uint32_t col_tiles, float t)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    const uint32_t i = threadIdx.x >> 6;
+    const uint64_t x = blockIdx.x / col_tiles;
+    const uint64_t y = (uint64_t)(blockIdx.x % col_tiles) * 256 + (uint64_t)lane * 4;
+    const uint64_t row = x * 16 + i;
+    if (row >= n || y >= k) return;
+    // with ALIGNED, k is a multiple of 4 and every lane inside the matrix owns 4 columns
+    const int cnt = ALIGNED ? 4 : ((k - y < 4) ? (int)(k - y) : 4);
+    const uint32_t sh = 2 * i;
+    const uint32_t* cw = c + x * k + y;
+    float* o = out + row * k + y;
+    // all 16 waves read the tile's 1 KiB of words (cache hits after the first)
+    if (cnt == 4) {
+        uint32_t w0, w1, w2, w3;
+        if constexpr (ALIGNED) {
+            const u32x4 w = *reinterpret_cast<const u32x4*>(cw);
+            w0 = w.x; w1 = w.y; w2 = w.z; w3 = w.w;
+        } else {
+            const u32x4_a4 w = *reinterpret_cast<const u32x4_a4*>(cw);
+            w0 = w.x; w1 = w.y; w2 = w.z; w3 = w.w;
+        }
+        f32x4 v;
+        v.x = deq_code((w0 >> sh) & 3u, t);
+        v.y = deq_code((w1 >> sh) & 3u, t);
+        v.z = deq_code((w2 >> sh) & 3u, t);
+        v.w = deq_code((w3 >> sh) & 3u, t);
+        st4<ALIGNED, NT>(o, v);
+    } else {
+        for (int j = 0; j < cnt; ++j) o[j] = deq_code((cw[j] >> sh) & 3u, t);
+    }
+}
+
+constexpr int kBlock2D = 256;  // workgroup size of the narrow-matrix kernels
+
+// Narrow matrices (k < 64 columns): a 256-column tile would leave most lanes idle, so one lane
+// takes one word and lanes walk along the flattened (x, y) index.
 template <bool ADD>
 __global__ __launch_bounds__(kBlock2D) void quant_2d_kernel(
     const float* g, const float* rin, float* rout, uint32_t* __restrict__ c, uint64_t n,
@@ -430,75 +543,6 @@ __global__ __launch_bounds__(kBlock2D) void deq_2d_kernel(float* out, const uint
             if (xm < n) out[xm * k + y] = deq_code((word >> (2 * i)) & 3u, t);
         }
     }
-}
-
-// Row-tiled matrix kernels, used when k % 4 == 0 and the bases are 16-byte aligned.  A
-// workgroup of 16 waves takes a tile of 16 rows x 256 columns: wave i moves row 16x+i of the
-// tile with one dwordx4 per lane (1 KiB contiguous, like a flat chunk), so neighbouring
-// workgroups (on different XCDs) touch neighbouring 1 KiB pieces of the same rows.  The 16 codes
-// of a word come from 16 different waves: each wave ORs its code, shifted to its bit position,
-// into the tile's 256 words in LDS; after a barrier 256 threads store the 1 KiB of words.
-constexpr int kRowsBlock = 16 * kWave;  // 1024 threads
-
-template <bool ADD, bool NT>
-__global__ __launch_bounds__(kRowsBlock) void quant_2d_rows_kernel(
-    const float* g, const float* rin, float* rout, uint32_t* __restrict__ c, uint64_t n,
-    uint64_t k, uint32_t col_tiles, float t)
-{
-    __shared__ uint32_t words[256];
-    const int lane = threadIdx.x & (kWave - 1);
-    const uint32_t i = threadIdx.x >> 6;  // row inside the tile = code position inside the word
-    const uint64_t x = blockIdx.x / col_tiles;
-    const uint64_t y0 = (uint64_t)(blockIdx.x % col_tiles) * 256;
-    const uint64_t y = y0 + (uint64_t)lane * 4;
-    const uint64_t row = x * 16 + i;
-    const bool live = row < n && y < k;
-    const uint64_t off = row * k + y;
-    f32x4 a = (f32x4)(0.0f), r = (f32x4)(0.0f);
-    if (live) {
-        a = ld4<true, NT>(g + off);
-        if constexpr (ADD) r = ld4<true, NT>(rin + off);
-    }
-    if (threadIdx.x < 256) words[threadIdx.x] = 0;
-    __syncthreads();
-    if (live) {
-        f32x4 v = a;
-        if constexpr (ADD) v = v + r;
-        float o0, o1, o2, o3;
-        const uint32_t c0 = quant_one(v.x, t, o0), c1 = quant_one(v.y, t, o1);
-        const uint32_t c2 = quant_one(v.z, t, o2), c3 = quant_one(v.w, t, o3);
-        f32x4 o;
-        o.x = o0; o.y = o1; o.z = o2; o.w = o3;
-        st4<true, NT>(rout + off, o);
-        const uint32_t sh = 2 * i;
-        if (c0) atomicOr(&words[lane * 4 + 0], c0 << sh);
-        if (c1) atomicOr(&words[lane * 4 + 1], c1 << sh);
-        if (c2) atomicOr(&words[lane * 4 + 2], c2 << sh);
-        if (c3) atomicOr(&words[lane * 4 + 3], c3 << sh);
-    }
-    __syncthreads();
-    if (threadIdx.x < 256 && y0 + threadIdx.x < k) c[x * k + y0 + threadIdx.x] = words[threadIdx.x];
-}
-
-template <bool NT>
-__global__ __launch_bounds__(kRowsBlock) void deq_2d_rows_kernel(
-    float* out, const uint32_t* __restrict__ c, uint64_t n, uint64_t k, uint32_t col_tiles, float t)
-{
-    const int lane = threadIdx.x & (kWave - 1);
-    const uint32_t i = threadIdx.x >> 6;
-    const uint64_t x = blockIdx.x / col_tiles;
-    const uint64_t y = (uint64_t)(blockIdx.x % col_tiles) * 256 + (uint64_t)lane * 4;
-    const uint64_t row = x * 16 + i;
-    if (row >= n || y >= k) return;
-    // all 16 waves read the tile's 1 KiB of words (cache hits after the first)
-    const u32x4 w = *reinterpret_cast<const u32x4*>(c + x * k + y);
-    const uint32_t sh = 2 * i;
-    f32x4 o;
-    o.x = deq_code((w.x >> sh) & 3u, t);
-    o.y = deq_code((w.y >> sh) & 3u, t);
-    o.z = deq_code((w.z >> sh) & 3u, t);
-    o.w = deq_code((w.w >> sh) & 3u, t);
-    st4<true, NT>(out + row * k + y, o);
 }
 
 // ---------------------------------------------------------------- many vectors in one launch
@@ -1045,25 +1089,7 @@ int nklq_quantize_f32(const float* g, const float* r_in, float* r_out, uint32_t*
         return dispatch_quant_flat(g, r_in, r_out, c, total, thrd, add, al, s);
     }
     const uint64_t m = n_rows / 16 + (n_rows % 16 ? 1 : 0);
-    const bool vec = (n_cols % 4 == 0) && aligned16(g) && aligned16(r_out) && aligned16(c) &&
-                     (!add || aligned16(r_in));
-    if (vec) {
-        const uint64_t col_tiles = (n_cols + 255) / 256;
-        const uint64_t tiles = m * col_tiles;
-        if (tiles > 0x7FFFFFFFull || col_tiles > 0xFFFFFFFFull) return NKLQ_ERANGE;
-        const dim3 grid((uint32_t)tiles), block(kRowsBlock);
-        const int sel = (add ? 2 : 0) | (g_nontemporal ? 1 : 0);
-#define NKLQ_Q2(ADD, NT)                                                                        \
-    hipLaunchKernelGGL((quant_2d_rows_kernel<ADD, NT>), grid, block, 0, s, g, r_in, r_out, c, n_rows, \
-                       n_cols, (uint32_t)col_tiles, thrd)
-        switch (sel) {
-            case 3: NKLQ_Q2(true, true); break;
-            case 2: NKLQ_Q2(true, false); break;
-            case 1: NKLQ_Q2(false, true); break;
-            default: NKLQ_Q2(false, false); break;
-        }
-#undef NKLQ_Q2
-    } else {
+    if (n_cols < kNarrowColumns) {
         const uint64_t items = m * n_cols;
         const uint32_t grid = grid_for_items(items);
         if (add)
@@ -1072,7 +1098,26 @@ int nklq_quantize_f32(const float* g, const float* r_in, float* r_out, uint32_t*
         else
             hipLaunchKernelGGL((quant_2d_kernel<false>), dim3(grid), dim3(kBlock2D), 0, s, g, r_in,
                                r_out, c, n_rows, n_cols, items, thrd);
+        return launch_status();
     }
+    const bool al = (n_cols % 4 == 0) && aligned16(g) && aligned16(r_out) && (!add || aligned16(r_in));
+    const uint64_t col_tiles = (n_cols + 255) / 256;
+    if (col_tiles > 0x7FFFFFFFull || m > 0x7FFFFFFFull / col_tiles) return NKLQ_ERANGE;
+    const dim3 grid((uint32_t)(m * col_tiles)), block(kRowsBlock);
+#define NKLQ_Q2(ADD, NT, AL)                                                                         \
+    hipLaunchKernelGGL((quant_2d_rows_kernel<ADD, NT, AL>), grid, block, 0, s, g, r_in, r_out, c, n_rows, \
+                       n_cols, (uint32_t)col_tiles, thrd)
+    switch ((add ? 4 : 0) | (g_nontemporal ? 2 : 0) | (al ? 1 : 0)) {
+        case 7: NKLQ_Q2(true, true, true); break;
+        case 6: NKLQ_Q2(true, true, false); break;
+        case 5: NKLQ_Q2(true, false, true); break;
+        case 4: NKLQ_Q2(true, false, false); break;
+        case 3: NKLQ_Q2(false, true, true); break;
+        case 2: NKLQ_Q2(false, true, false); break;
+        case 1: NKLQ_Q2(false, false, true); break;
+        default: NKLQ_Q2(false, false, false); break;
+    }
+#undef NKLQ_Q2
     return launch_status();
 }
 
@@ -1090,21 +1135,24 @@ int nklq_dequantize_f32(float* out, const uint32_t* c, uint64_t n_rows, uint64_t
         return dispatch_deq_flat(out, c, total, thrd, s);
     }
     const uint64_t m = n_rows / 16 + (n_rows % 16 ? 1 : 0);
-    if ((n_cols % 4 == 0) && aligned16(out) && aligned16(c)) {
-        const uint64_t col_tiles = (n_cols + 255) / 256;
-        const uint64_t tiles = m * col_tiles;
-        if (tiles > 0x7FFFFFFFull || col_tiles > 0xFFFFFFFFull) return NKLQ_ERANGE;
-        if (g_nontemporal)
-            hipLaunchKernelGGL((deq_2d_rows_kernel<true>), dim3((uint32_t)tiles), dim3(kRowsBlock), 0, s,
-                               out, c, n_rows, n_cols, (uint32_t)col_tiles, thrd);
-        else
-            hipLaunchKernelGGL((deq_2d_rows_kernel<false>), dim3((uint32_t)tiles), dim3(kRowsBlock), 0,
-                               s, out, c, n_rows, n_cols, (uint32_t)col_tiles, thrd);
-    } else {
+    if (n_cols < kNarrowColumns) {
         const uint64_t items = m * n_cols;
-        hipLaunchKernelGGL((deq_2d_kernel), dim3(grid_for_items(items)), dim3(kBlock2D), 0, s, out,
-                           c, n_rows, n_cols, items, thrd);
+        hipLaunchKernelGGL((deq_2d_kernel), dim3(grid_for_items(items)), dim3(kBlock2D), 0, s, out, c,
+                           n_rows, n_cols, items, thrd);
+        return launch_status();
     }
+    const bool al = (n_cols % 4 == 0) && aligned16(out) && aligned16(c);
+    const uint64_t col_tiles = (n_cols + 255) / 256;
+    if (col_tiles > 0x7FFFFFFFull || m > 0x7FFFFFFFull / col_tiles) return NKLQ_ERANGE;
+    const dim3 grid((uint32_t)(m * col_tiles)), block(kRowsBlock);
+#define NKLQ_D2(NT, AL)                                                                            \
+    hipLaunchKernelGGL((deq_2d_rows_kernel<NT, AL>), grid, block, 0, s, out, c, n_rows, n_cols, \
+                       (uint32_t)col_tiles, thrd)
+    if (g_nontemporal && al) NKLQ_D2(true, true);
+    else if (g_nontemporal) NKLQ_D2(true, false);
+    else if (al) NKLQ_D2(false, true);
+    else NKLQ_D2(false, false);
+#undef NKLQ_D2
     return launch_status();
 }
 
