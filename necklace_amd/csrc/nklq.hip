@@ -1169,6 +1169,11 @@ int nklq_dequant_accumulate_f32(float* acc, const uint32_t* const* payloads, int
         if ((const void*)payloads[p] == (const void*)acc) return NKLQ_EALIAS;
     }
     hipStream_t s = (hipStream_t)stream;
+    if (k_payloads == 1 && !accumulate && (__builtin_bit_cast(uint32_t, thrd) & 0x7FFFFFFFu) != 0) {
+        // +0.0 + d is d for d in {+t, -t, +0.0} unless t is a zero (then -t = -0.0 would become
+        // +0.0): a single payload into a fresh buffer is the plain decode, which is faster
+        return dispatch_deq_flat(acc, payloads[0], n, thrd, s);
+    }
     int acc_flag = accumulate ? 1 : 0;
     for (int first = 0; first < k_payloads; first += NKLQ_MAX_PAYLOADS_PER_LAUNCH) {
         PayloadPtrs pl = {};

@@ -283,3 +283,54 @@ def test_many_vectors_in_one_launch(knobs):
         pl = [msgs[k, woffs[i]:woffs[i] + (n + 15) // 16].copy() for k in range(K)]
         want = (oracle.c.dequant_accumulate(pl, n, thrd) / np.float32(7.0)).astype(np.float32)
         assert_bits_equal(accs[i].cpu().numpy(), want, f"vector {i} n={n} divided")
+
+
+def test_two_host_threads_on_two_streams():
+    """The library keeps no per-call state: two host threads driving two streams at once get the
+    same bits as one after the other."""
+    import threading
+    rng = np.random.default_rng(55)
+    n = 3_000_000 + 5
+    work = []
+    for i in range(2):
+        g = rng.normal(0, 1e-3, n).astype(np.float32)
+        r = rng.normal(0, 5e-4, n).astype(np.float32)
+        work.append((g, r, oracle.c.quantize(g, 1e-3, R_in=r)))
+    results, errors = [None, None], []
+
+    def run(i):
+        try:
+            torch.cuda.set_device(0)
+            s = torch.cuda.Stream()
+            with torch.cuda.stream(s):
+                dg, dr, dc = dev(work[i][0]), dev(work[i][1]), words_like(n)
+                for _ in range(20):  # keep both streams busy at the same time
+                    dr.copy_(dev(work[i][1]))
+                    q.cu_fn_matrix_quantize_e(dg, dc, dr, 1e-3, add_residual=True, stream=s, sync=False)
+                s.synchronize()
+                results[i] = (host_words(dc), dr.cpu().numpy())
+        except Exception as exc:  # surfaced below, in the main thread
+            errors.append(exc)
+
+    threads = [threading.Thread(target=run, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for i in range(2):
+        assert_words_equal(results[i][0], work[i][2][0], f"thread {i}")
+        assert_bits_equal(results[i][1], work[i][2][1], f"thread {i}")
+
+
+def test_empty_inputs_are_no_ops():
+    e = torch.empty(0, device="cuda")
+    w = torch.empty(0, dtype=torch.int32, device="cuda")
+    q.cu_fn_matrix_quantize_e(e, w, e.clone(), 0.5)
+    q.cu_fn_matrix_dequantize_e(e, w, None, 0.5)
+    q.cu_fn_dequantize_accumulate_e(e, [w], 0.5)
+    q.cu_fn_quantize_multi_e([e], [w], [e.clone()], 0.5)
+    q.cu_fn_quantize_multi_e([], [], [], 0.5)
+    m = torch.empty(0, 7, device="cuda")
+    q.cu_fn_matrix_quantize_e(m, torch.empty(0, 7, dtype=torch.int32, device="cuda"), m.clone(), 0.5)
+    torch.cuda.synchronize()
