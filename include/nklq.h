@@ -102,7 +102,7 @@ int nklq_dequant_accumulate_f32(float* acc, const uint32_t* const* payloads, int
                                 uint64_t n, float thrd, int accumulate, void* stream);
 
 /*
- * The two flat operations above on MANY vectors with one launch per 32 of them: a model's
+ * The two flat operations above on MANY vectors with one launch per 96 of them: a model's
  * gradients are a list of separate tensors, and the per-parameter lists grd_resi / grd_comp /
  * grd_recv that necklace's trainer keeps (necklace/trainer/tnopmx.py:140-149) are lists of
  * separate buffers.  All array arguments are HOST arrays of `count` entries, read during the

@@ -549,10 +549,10 @@ __global__ __launch_bounds__(kBlock2D) void deq_2d_kernel(float* out, const uint
 
 // A model's gradients are many separate vectors (161 for ResNet-50, most of them small); one
 // launch per vector costs more in launch latency than the data takes to stream.  These kernels
-// take a table of up to kMaxSegments vectors in their arguments and treat the chunks (or tiles)
+// take a table of up to kMaxSegments (96) vectors in their arguments and treat the chunks (or tiles)
 // of all of them as one index space; a wave finds its vector by binary search in the table.
 
-constexpr int kMaxSegments = 32;
+constexpr int kMaxSegments = 96;  // 96 x 36 B of table stays under the 4 KiB kernel-argument limit
 
 struct QuantSegments {
     const float* g[kMaxSegments];

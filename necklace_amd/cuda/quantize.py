@@ -221,7 +221,7 @@ def _ptr_array(ptrs):
 
 
 def cu_fn_quantize_multi_e(grads, comps, resis, thrd=0.3, add_residual=True, stream=None, sync=True):
-    """Flat quantize of many vectors with one launch per 32 of them.
+    """Flat quantize of many vectors with one launch per 96 of them.
 
     ``grads[i]``, ``resis[i]``: float32 GPU tensors of the same number of elements (any shape,
     contiguous); ``comps[i]``: ceil(numel/16) words.  With ``add_residual`` the residual is read,
@@ -256,7 +256,7 @@ def cu_fn_quantize_multi_e(grads, comps, resis, thrd=0.3, add_residual=True, str
 
 def cu_fn_dequantize_accumulate_multi_e(accs, word_offsets, payloads, thrd=0.3, accumulate=False,
                                         divisor=1.0, stream=None, sync=True):
-    """Fixed-order decode-and-sum into many vectors with one launch per 32 of them.
+    """Fixed-order decode-and-sum into many vectors with one launch per 96 of them.
 
     ``payloads``: one 2-D tensor [K, W] (or a list of K 1-D tensors of W words): the message of
     each of the K peers.  Vector i (``accs[i]``, float32, contiguous) has its code words at

@@ -153,7 +153,7 @@ class GradCompressor:
         """Quantize every compressed parameter's gradient with error feedback.
 
         `grads[i]` is parameter i's gradient (any shape, contiguous fp32 on the GPU);
-        entries of uncompressed parameters are ignored.  One launch per 32 parameters.
+        entries of uncompressed parameters are ignored.  One launch per 96 parameters.
         """
         g_arr = self._ptrs(grads, "gradient")
         if not self._idx:

@@ -229,9 +229,9 @@ def test_round_trip_and_zero_residual_on_gpu():
 
 
 def test_many_vectors_in_one_launch(knobs):
-    """nklq_quantize_multi_f32 / nklq_dequant_accumulate_multi_f32: 45 vectors of awkward lengths
-    (more than one table of 32), some at odd element offsets, each equal to its own flat result."""
-    sizes = [1, 15, 16, 17, 255, 256, 257, 511, 1023, 1024, 1025, 2047, 4096, 5000, 70001] * 3
+    """nklq_quantize_multi_f32 / nklq_dequant_accumulate_multi_f32: 105 vectors of awkward lengths
+    (more than one table of 96), some at odd element offsets, each equal to its own flat result."""
+    sizes = [1, 15, 16, 17, 255, 256, 257, 511, 1023, 1024, 1025, 2047, 4096, 5000, 70001] * 7
     rng = np.random.default_rng(314)
     thrd, K = 1e-3, 3
     arena_g = torch.zeros(sum(sizes) + 4 * len(sizes), device="cuda")
@@ -258,7 +258,7 @@ def test_many_vectors_in_one_launch(knobs):
     # plain form: residual only written
     outs = [torch.full((n,), 3.0, device="cuda") for n in sizes]
     q.cu_fn_quantize_multi_e(grads, comps, outs, thrd, add_residual=False)
-    for i in (0, 4, 9, 14, 44):
+    for i in (0, 4, 9, 14, 44, 95, 96, 104):
         want_c, want_r = oracle.c.quantize(gh[i], thrd)
         assert_words_equal(host_words(comps[i]), want_c)
         assert_bits_equal(outs[i].cpu().numpy(), want_r)
