@@ -17,12 +17,15 @@
 //     together with two DPP quad permutes (no LDS, no memory) to form the word of
 //     16 codes;
 //   * the residual is written back in the same pass (one read of g and r, one
-//     write of r and of the codes: 12.25 bytes per element); loads and stores
-//     are non-temporal, the data is touched once;
+//     write of r and of the codes: 12.25 bytes per element); the fp32 streams
+//     use non-temporal loads and stores (touched once), the code words ordinary
+//     ones (two chunks share a 128 B line of them);
 //   * the last partial chunk goes through a bounds-checked one-element-per-lane
 //     path in one extra workgroup of the same launch (codes combined across the
 //     16 lanes of a DPP row);
-//   * 64-bit element indices throughout (vectors of more than 2^31 elements).
+//   * 64-bit element indices throughout (vectors of more than 2^31 elements);
+//   * the sum over K payloads (acc_flat_kernel), the matrix form (quant_2d_rows_kernel) and
+//     the many-vectors form (quant_multi_kernel) are described at their kernels.
 //
 // fp32 arithmetic is IEEE: no fast-math, no contraction, denormals kept.
 #include <hip/hip_runtime.h>
