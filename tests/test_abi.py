@@ -80,3 +80,19 @@ def test_tune_knobs_round_trip():
         _lib.tune(which, before)
     with pytest.raises(ValueError):
         _lib.tune(9, 1)
+
+
+def test_missing_library_is_an_error_not_a_fallback(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "SO_PATH", str(tmp_path / "libnklq.so"))
+    with pytest.raises(ImportError):
+        _lib.lib()
+
+
+def test_the_package_never_touches_the_cpu_checker():
+    pkg = os.path.join(ROOT, "necklace_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text, f"{f} mentions the checker"
