@@ -124,6 +124,9 @@ def main():
         print("bench.py: this path runs on ONE GPU (no collectives are part of it); "
               "use --gpus 1", file=sys.stderr)
         sys.exit(2)
+    if args.chunk < 0 or args.chunk % 16:
+        print("bench.py: --chunk must be a non-negative multiple of 16", file=sys.stderr)
+        sys.exit(2)
 
     import torch
     from necklace_amd.csrc import build as hip_build
@@ -145,9 +148,6 @@ def main():
     c = torch.empty(_lib.packed_words(n), dtype=torch.int32, device="cuda")
     stream = torch.cuda.current_stream().cuda_stream
 
-    if args.chunk < 0 or args.chunk % 16:
-        print("bench.py: --chunk must be a non-negative multiple of 16", file=sys.stderr)
-        sys.exit(2)
     chunk = args.chunk or n
     pieces = [(lo, min(n, lo + chunk)) for lo in range(0, n, chunk)]
     gp, rp, cp = g.data_ptr(), r.data_ptr(), c.data_ptr()
