@@ -48,12 +48,12 @@ def _shape2(t):
     return t.shape[0], t.shape[1]
 
 
-def _check_f32(name, t):
+def _check_f32(name, t, any_rank=False):
     if not isinstance(t, torch.Tensor):
         raise TypeError(f"{name}: expected a torch tensor, got {type(t).__name__}")
     if t.dtype != torch.float32:
         raise TypeError(f"{name}: expected float32, got {t.dtype}")
-    if t.dim() not in (1, 2):
+    if not any_rank and t.dim() not in (1, 2):
         raise TypeError(f"{name}: expected 1 or 2 dimensions, got {t.dim()}")
     if not t.is_cuda:
         raise TypeError(f"{name}: expected a GPU tensor (pass to_device=True for host arrays)")
@@ -236,8 +236,8 @@ def cu_fn_quantize_multi_e(grads, comps, resis, thrd=0.3, add_residual=True, str
     dev = grads[0].device
     ns = []
     for i, (gr, cm, rs) in enumerate(zip(grads, comps, resis)):
-        _check_f32(f"grads[{i}]", gr.reshape(-1) if isinstance(gr, torch.Tensor) and gr.dim() > 2 else gr)
-        _check_f32(f"resis[{i}]", rs.reshape(-1) if isinstance(rs, torch.Tensor) and rs.dim() > 2 else rs)
+        _check_f32(f"grads[{i}]", gr, any_rank=True)
+        _check_f32(f"resis[{i}]", rs, any_rank=True)
         n = gr.numel()
         if rs.numel() != n:
             raise ValueError(f"resis[{i}] has {rs.numel()} elements, grads[{i}] has {n}")
@@ -282,7 +282,7 @@ def cu_fn_dequantize_accumulate_multi_e(accs, word_offsets, payloads, thrd=0.3, 
             raise ValueError(f"payloads[{i}]: must be contiguous, on the same GPU and of equal length")
     ns = []
     for i, (a, wo) in enumerate(zip(accs, word_offsets)):
-        _check_f32(f"accs[{i}]", a.reshape(-1) if isinstance(a, torch.Tensor) and a.dim() > 2 else a)
+        _check_f32(f"accs[{i}]", a, any_rank=True)
         if a.device != dev:
             raise ValueError("all tensors must be on the same GPU")
         n = a.numel()
