@@ -197,6 +197,10 @@ def main():
             "thrd": THRD,
             "layout": "flat (N,1): word w packs elements 16w..16w+15",
             "launches_per_step": len(pieces),
+            "launch_geometry": {"chunks_per_wave": _lib.tune(_lib.TUNE_CHUNKS_PER_WAVE),
+                                "workgroup": _lib.tune(_lib.TUNE_WORKGROUP_SIZE),
+                                "nontemporal": _lib.tune(_lib.TUNE_NONTEMPORAL),
+                                "xcd_interleave_log2": _lib.tune(_lib.TUNE_XCD_INTERLEAVE_LOG2)},
         },
         "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
         "roofline": {
