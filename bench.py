@@ -166,6 +166,15 @@ def main():
     value = BYTES_QUANT * n / (ms_per_step * 1e-3) / 1e9
     achieved = bytes_per_launch / (kernel_ms * 1e-3) / 1e9
 
+    # spread of single steps (outside the timed region): one event pair per step
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(30)]
+    for e0, e1 in pairs:
+        e0.record()
+        step()
+        e1.record()
+    torch.cuda.synchronize()
+    singles = sorted(e0.elapsed_time(e1) for e0, e1 in pairs)
+
     traffic = None
     tpath = os.path.join(ROOT, "profiles", "traffic.json")
     if os.path.exists(tpath) and n == N_ELEMS:
@@ -214,6 +223,8 @@ def main():
             "bytes_per_launch": bytes_per_launch,
             "avg_launch_ms": round(kernel_ms, 4),
         },
+        "single_step_ms": {"median": round(singles[len(singles) // 2], 4), "min": round(singles[0], 4),
+                           "max": round(singles[-1], 4), "samples": len(singles)},
     }
 
     legs = {x for x in args.legs.split(",") if x}
