@@ -321,3 +321,105 @@ def load_grad_comp_state(grad_comp_cfg, state):
     """Restore what `grad_comp_state` saved into a `grad_comp_cfg` built for the same parameters."""
     grad_comp_cfg["compressor"].load_state_dict(state)
     grad_comp_cfg["grad_comp_threshold"] = float(state["thrd"])
+
+
+# --------------------------------------------------------------------------- ptprms call surface
+
+def _opt_grads(opt):
+    """The gradients an optimizer owns, in the order necklace walks them
+    (necklace/frmwrk/pytorch/ptprms.py:331-336)."""
+    grads = []
+    for group in opt.param_groups:
+        for p in group["params"]:
+            if p.grad is not None:
+                grads.append(p.grad.data)
+    return grads
+
+
+def _exchange_of(nc):
+    """`nc` stands where necklace passes its NCCL communicator.  Collectives are not part of this
+    package, so it is whatever gathers the payloads: a callable ``nc(comp, recv)`` or an object
+    with ``all_gather_words(comp, recv)``; None is allowed for a single worker."""
+    if nc is None or callable(nc):
+        return nc
+    return nc.all_gather_words
+
+
+def _cfg_for(grads, kn, grad_comp_cfg):
+    if grad_comp_cfg is None:
+        raise ValueError("grad_comp_cfg is required: this is the compressed path")
+    if "compressor" not in grad_comp_cfg:
+        # first call: lay the buffers out for these gradients (trainer/tnopmx.py:135-151 does this
+        # once at set-up; doing it lazily here keeps the call sites of ptprms unchanged)
+        built = init_grad_comp_cfg(grads, kn, grad_comp_cfg, device=grads[0].device,
+                                   rank=grad_comp_cfg.get("rank", 0))
+        grad_comp_cfg.update(built)
+    return grad_comp_cfg
+
+
+def opt_one_grads_do_nccl_allreduce(nc, kn, opt, prm_revs=None, grad_comp_cfg=None):
+    """Compressed counterpart of ptprms.opt_one_grads_do_nccl_allreduce
+    (necklace/frmwrk/pytorch/ptprms.py:329-338): every gradient of at least
+    ``grad_size_threshold`` elements is replaced by the average over the `kn` workers of its 2-bit
+    decode.  Returns the gradients below the threshold: they still need the ordinary all-reduce."""
+    grads = _opt_grads(opt)
+    if not grads:
+        return []
+    cfg = _cfg_for(grads, kn, grad_comp_cfg)
+    small = grads_do_compressed_exchange(grads, kn, cfg, exchange=_exchange_of(nc), average=True)
+    return [grads[i] for i in small]
+
+
+def opt_grads_do_nccl_allreduce(nc, kn, opt, prm_revs=None, grad_comp_cfg=None):
+    """ptprms.opt_grads_do_nccl_allreduce (ptprms.py:319-326): one optimizer or a list of them, each
+    with its own ``grad_comp_cfg`` entry when a list of configs is given."""
+    if isinstance(opt, (list, tuple)):
+        cfgs = grad_comp_cfg if isinstance(grad_comp_cfg, (list, tuple)) else [grad_comp_cfg] * len(opt)
+        if len(opt) > 1 and not isinstance(grad_comp_cfg, (list, tuple)):
+            raise ValueError("several optimizers need one grad_comp_cfg each (their residuals differ)")
+        out = []
+        for o, c in zip(opt, cfgs):
+            out += opt_one_grads_do_nccl_allreduce(nc, kn, o, prm_revs=prm_revs, grad_comp_cfg=c)
+        return out
+    return opt_one_grads_do_nccl_allreduce(nc, kn, opt, prm_revs=prm_revs, grad_comp_cfg=grad_comp_cfg)
+
+
+def opt_grads_do_nccl_reduce(nc, kn, root, opt, prm_revs=None, grad_comp_cfg=None):
+    """Compressed counterpart of ptprms.opt_grads_do_nccl_reduce (ptprms.py:344-363): like the
+    all-reduce but only worker `root` decodes, and the sum is not averaged (the reference's reduce
+    leaves the `/ kn` commented out, ptprms.py:385)."""
+    grads = _opt_grads(opt)
+    if not grads:
+        return []
+    cfg = _cfg_for(grads, kn, grad_comp_cfg)
+    gc = cfg["compressor"]
+    if gc.kn != kn:
+        raise ValueError(f"grad_comp_cfg was built for kn={gc.kn}, got kn={kn}")
+    gc.compress(grads)
+    exchange = _exchange_of(nc)
+    if exchange is not None:
+        exchange(gc.comp, gc.recv)
+    elif kn != 1:
+        raise ValueError("an exchange is required when kn > 1")
+    if gc.rank == root:
+        gc.decompress_sum(grads, average=False)
+    return [grads[i] for i, c in enumerate(gc.grd_cmps) if not c]
+
+
+def opt_grads_fltn_do_nccl_reduce(nc, kn, root, d_arr_send, sz, grad_comp_cfg=None):
+    """Compressed counterpart of ptprms.opt_grads_fltn_do_nccl_reduce (ptprms.py:396-401) on the
+    flat gradient buffer; see `opt_grads_fltn_do_compressed_reduce`.  Only `root` decodes."""
+    if grad_comp_cfg is None or "compressor" not in grad_comp_cfg:
+        raise ValueError("build grad_comp_cfg with init_flat_grad_comp_cfg first")
+    gc = grad_comp_cfg["compressor"]
+    if gc.kn != kn:
+        raise ValueError(f"grad_comp_cfg was built for kn={gc.kn}, got kn={kn}")
+    flat = d_arr_send.reshape(-1)[:sz]
+    gc.compress_flat(flat)
+    exchange = _exchange_of(nc)
+    if exchange is not None:
+        exchange(gc.comp, gc.recv)
+    elif kn != 1:
+        raise ValueError("an exchange is required when kn > 1")
+    if gc.rank == root:
+        gc.decompress_sum([flat], average=False)

@@ -139,3 +139,46 @@ def test_checkpoint_file_round_trip(tmp_path):
     assert cfg2["compressor"].thrd == thrd
     assert torch.equal(cfg2["compressor"].resi.view(torch.int32), cfg["compressor"].resi.view(torch.int32))
     assert state["epoch"] == 3
+
+
+def test_ptprms_call_surface_on_a_real_optimizer():
+    """opt_grads_do_nccl_allreduce / _reduce with necklace's argument order on the gradients of a
+    small MLP (the shape of the reference's MNIST example), two workers whose payloads coincide."""
+    torch.manual_seed(0)
+    model = torch.nn.Sequential(torch.nn.Linear(784, 256), torch.nn.ReLU(), torch.nn.Linear(256, 64),
+                                torch.nn.ReLU(), torch.nn.Linear(64, 10)).cuda()
+    opt = torch.optim.SGD(model.parameters(), lr=0.1)
+    x = torch.randn(32, 784, device="cuda")
+    loss = torch.nn.functional.cross_entropy(model(x), torch.randint(0, 10, (32,), device="cuda"))
+    loss.backward()
+    thrd, kn = 1e-3, 2
+    before = [p.grad.detach().cpu().numpy().copy() for p in model.parameters()]
+
+    def same_payload_from_both(comp, recv):
+        recv[1].copy_(recv[0])
+
+    cfg = {"grad_comp_threshold": thrd, "grad_size_threshold": 1001}
+    small = ptcomp.opt_grads_do_nccl_allreduce(same_payload_from_both, kn, opt, None, grad_comp_cfg=cfg)
+    torch.cuda.synchronize()
+    assert "compressor" in cfg
+    sizes = [g.size for g in before]
+    assert sorted(t.numel() for t in small) == sorted(s for s in sizes if s < 1001)
+    for p, g in zip(model.parameters(), before):
+        got = p.grad.detach().cpu().numpy()
+        if g.size < 1001:
+            assert_bits_equal(got, g, "small gradients are left to the ordinary all-reduce")
+            continue
+        c, _ = oracle.c.quantize(g.reshape(-1), thrd, R_in=np.zeros(g.size, np.float32))
+        want = (oracle.c.dequant_accumulate([c, c], g.size, thrd) / np.float32(kn)).astype(np.float32)
+        assert_bits_equal(got.reshape(-1), want, f"gradient of {g.shape}")
+    # reduce-to-root: the non-root worker compresses and sends but keeps its gradient
+    cfg1 = {"grad_comp_threshold": thrd, "rank": 1}
+    loss = torch.nn.functional.cross_entropy(model(x), torch.randint(0, 10, (32,), device="cuda"))
+    opt.zero_grad(set_to_none=False)
+    loss.backward()
+    keep = [p.grad.detach().clone() for p in model.parameters()]
+    ptcomp.opt_grads_do_nccl_reduce(lambda comp, recv: None, kn, 0, opt, None, grad_comp_cfg=cfg1)
+    torch.cuda.synchronize()
+    for p, k in zip(model.parameters(), keep):
+        assert torch.equal(p.grad, k)
+    assert int((cfg1["compressor"].comp != 0).sum()) > 0
