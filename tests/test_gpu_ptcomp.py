@@ -182,3 +182,25 @@ def test_ptprms_call_surface_on_a_real_optimizer():
     for p, k in zip(model.parameters(), keep):
         assert torch.equal(p.grad, k)
     assert int((cfg1["compressor"].comp != 0).sum()) > 0
+
+
+def test_sgd_with_compressed_gradients_still_learns():
+    """End to end on one worker: every step's gradients go through compress -> decompress (2 bits
+    per element plus error feedback) before the optimizer sees them, and the model still fits."""
+    torch.manual_seed(1)
+    x = torch.randn(512, 64, device="cuda")
+    w_true = torch.randn(64, 10, device="cuda")
+    y = (x @ w_true).argmax(1)
+    model = torch.nn.Sequential(torch.nn.Linear(64, 128), torch.nn.ReLU(), torch.nn.Linear(128, 10)).cuda()
+    opt = torch.optim.SGD(model.parameters(), lr=0.2)
+    cfg = {"grad_comp_threshold": 2e-3, "grad_size_threshold": 1}
+    losses = []
+    for step in range(150):
+        opt.zero_grad(set_to_none=False)
+        loss = torch.nn.functional.cross_entropy(model(x), y)
+        loss.backward()
+        ptcomp.opt_grads_do_nccl_allreduce(None, 1, opt, None, grad_comp_cfg=cfg)
+        opt.step()
+        losses.append(float(loss))
+    assert losses[-1] < 0.5 * losses[0], (losses[0], losses[-1])
+    assert bool(torch.isfinite(cfg["compressor"].resi).all())
