@@ -275,6 +275,28 @@ def main():
             "ms": round(acc_ms, 4),
             "GBps": round(acc_bytes / (acc_ms * 1e-3) / 1e9, 1),
         }
+        del payloads, acc
+        # the same sum at gradient size: 8 random payloads (the kernel's time does not depend on the codes)
+        if n >= 1 << 24:
+            wl = _lib.packed_words(n)
+            big = torch.randint(-2 ** 31, 2 ** 31 - 1, (K_PAYLOADS, wl), dtype=torch.int32, device="cuda",
+                                generator=gen)
+            accl = torch.empty(n, dtype=torch.float32, device="cuda")
+            ptrl = (ct.c_void_p * K_PAYLOADS)(*[big[p].data_ptr() for p in range(K_PAYLOADS)])
+
+            def accum_large():
+                _lib.check(L.nklq_dequant_accumulate_f32(accl.data_ptr(), ptrl, K_PAYLOADS, n, THRD, 0, stream))
+
+            for _ in range(3):
+                accum_large()
+            _, ev = time_region(torch, accum_large, 20)
+            res["dequant_accumulate_large"] = {
+                "payloads": K_PAYLOADS, "elements": n,
+                "elements_per_s": round(n / (ev / 20 * 1e-3)),
+                "ms": round(ev / 20, 4),
+                "GBps": round((0.25 * K_PAYLOADS + 4) * n / (ev / 20 * 1e-3) / 1e9, 1),
+            }
+            del big, accl
 
     if "matrix" in legs:
         # the reference's own layout: (n, k) matrix, codes packed down the columns
