@@ -175,13 +175,15 @@ def main():
     torch.cuda.synchronize()
     singles = sorted(e0.elapsed_time(e1) for e0, e1 in pairs)
 
+    # HBM bytes per launch from the rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this same command
+    # (a separate, committed measurement: counters cannot be read from inside the process)
     traffic = None
-    tpath = os.path.join(ROOT, "profiles", "traffic.json")
-    if os.path.exists(tpath) and n == N_ELEMS:
-        try:
-            traffic = json.load(open(tpath)).get("quant_flat_bytes_per_launch")
-        except Exception:
-            traffic = None
+    tpath = os.path.join(ROOT, "profiles", "quant_flat_355M_pmc.txt")
+    if os.path.exists(tpath) and n == N_ELEMS and len(pieces) == 1:
+        import re
+        m = re.search(r"^\s*total\s+([0-9,]+) B\s+vs algorithmic", open(tpath).read(), re.M)
+        if m:
+            traffic = int(m.group(1).replace(",", ""))
 
     res = {
         "metric": "fused 2-bit quantize GB/s (355M fp32 grad)" if n == N_ELEMS
