@@ -334,3 +334,31 @@ def test_empty_inputs_are_no_ops():
     m = torch.empty(0, 7, device="cuda")
     q.cu_fn_matrix_quantize_e(m, torch.empty(0, 7, dtype=torch.int32, device="cuda"), m.clone(), 0.5)
     torch.cuda.synchronize()
+
+
+def test_nbutils_helpers_and_kernel_object_decode():
+    """The device helpers of necklace/cuda/nbutils.py:11-39 on torch, and the subscripted decode
+    kernel (necklace/cuda/quantize.py:134)."""
+    from necklace_amd.cuda import nbutils
+    nbutils.cuda_select_device(0)
+    assert nbutils.cuda_current_context() == torch.device("cuda", 0)
+    s = nbutils.cuda_stream()
+    rng = np.random.default_rng(9)
+    n = 64
+    A = (rng.random((n, n)).astype(np.float32) - np.float32(1.0))
+    dA = nbutils.cuda_to_device(A, s)
+    dC = nbutils.cuda_to_device(np.zeros((4, n), np.uint32), s)
+    dR = nbutils.cuda_to_device(np.empty_like(A), s)
+    s.synchronize()
+    assert nbutils.cuda_devarr_c_void_p(dA).value == dA.data_ptr()
+    q.cu_knl_matrix_quantize_e[(4, 4), (8, 128), s](dA, dC, dR, 0.5)
+    dB = torch.empty(n, n, device="cuda")
+    q.cu_knl_matrix_dequantize_e[(4, 4), (8, 128), s](dB, dC, dR, 0.5)
+    s.synchronize()
+    want_c, want_r = oracle.c.quantize(A, 0.5)
+    assert_words_equal(host_words(dC), want_c)
+    assert_bits_equal(dR.cpu().numpy(), want_r)
+    assert_bits_equal(dB.cpu().numpy(), oracle.c.dequantize(want_c, n, 0.5))
+    # to_device=True decode from host arrays
+    hB, hC, _ = q.cu_fn_matrix_dequantize_e(np.empty_like(A), want_c, None, 0.5, to_device=True)
+    assert_bits_equal(hB.cpu().numpy(), oracle.c.dequantize(want_c, n, 0.5))
