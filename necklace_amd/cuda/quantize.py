@@ -297,3 +297,33 @@ def cu_fn_dequantize_accumulate_multi_e(accs, word_offsets, payloads, thrd=0.3, 
             _ptr_array([p.data_ptr() for p in payloads]), len(payloads), float(thrd),
             1 if accumulate else 0, float(divisor), h))
         _finish(stream, dev, sync)
+
+
+# ------------------------------------------------------------------ the reference's own smoke
+
+def test_11():
+    """The timing smoke of necklace/cuda/quantize.py:139-174 on this implementation: a 224 x 224
+    matrix of values in [-1, 0), thrd 0.5, quantize then dequantize, wall time of each printed."""
+    from timeit import default_timer as time
+
+    n = 7 * 32
+    m = packed_rows(n)
+    thrd = 0.5
+    A = torch.rand(n, n, device="cuda") - thrd * 2
+    R = torch.empty_like(A)
+    C = torch.zeros(m, n, dtype=torch.int32, device="cuda")
+    torch.cuda.synchronize()
+
+    tm = time()
+    cu_fn_matrix_quantize_e(A, C, R, thrd)
+    print('quantize: ', time() - tm)
+
+    B = torch.empty_like(A)
+    tm = time()
+    cu_fn_matrix_dequantize_e(B, C, R, thrd)
+    print('dequantize: ', time() - tm)
+    return A, B, C, R
+
+
+if __name__ == '__main__':
+    test_11()

@@ -362,3 +362,13 @@ def test_nbutils_helpers_and_kernel_object_decode():
     # to_device=True decode from host arrays
     hB, hC, _ = q.cu_fn_matrix_dequantize_e(np.empty_like(A), want_c, None, 0.5, to_device=True)
     assert_bits_equal(hB.cpu().numpy(), oracle.c.dequantize(want_c, n, 0.5))
+
+
+def test_the_reference_smoke_runs_and_is_consistent(capsys):
+    A, B, C, R = q.test_11()
+    out = capsys.readouterr().out
+    assert "quantize:" in out and "dequantize:" in out
+    want_c, want_r = oracle.c.quantize(A.cpu().numpy(), 0.5)
+    assert_words_equal(host_words(C), want_c)
+    assert_bits_equal(R.cpu().numpy(), want_r)
+    assert_bits_equal(B.cpu().numpy(), oracle.c.dequantize(want_c, 224, 0.5))
