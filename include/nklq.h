@@ -149,7 +149,8 @@ int nklq_version(void);
 #define NKLQ_TUNE_NONTEMPORAL 2          /* non-temporal loads and stores of the fp32 streams: 0 or 1 */
 #define NKLQ_TUNE_XCD_INTERLEAVE_LOG2 3  /* quantize: neighbouring chunks are dealt to 2^v consecutive
                                             workgroups (which run on different XCDs): 0..6 */
-#define NKLQ_TUNE_XCD_INTERLEAVE_LOG2_DECODE 4  /* the same for dequantize / accumulate */
+#define NKLQ_TUNE_XCD_INTERLEAVE_LOG2_DECODE 4  /* the same for dequantize */
+#define NKLQ_TUNE_XCD_INTERLEAVE_LOG2_ACCUMULATE 5  /* the same for the tiles (1024 elements) of the sum over payloads */
 int nklq_tune(int which, int value);
 
 /*

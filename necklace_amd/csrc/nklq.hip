@@ -260,78 +260,77 @@ struct PayloadPtrs {
     const uint32_t* p[NKLQ_MAX_PAYLOADS_PER_LAUNCH];
 };
 
-constexpr int kTile = 1024;        // elements per wave in the accumulate kernel: 64 code words
-constexpr int kLdsLaneStride = 20; // floats per lane in LDS (16 used): keeps b128 accesses off shared banks
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 
-// Position in a wave's LDS area of element `idx` (0..1023) of the tile.
-__device__ __forceinline__ int lds_pos(int idx) { return kLdsLaneStride * (idx >> 4) + (idx & 15); }
+constexpr int kTile = 1024;          // elements per wave in the accumulate kernels: 64 code words
+constexpr int kAccBlock = 256;       // 4 waves, 4 tiles per workgroup
+constexpr int kAccLdsPerWave = 1024; // LDS floats per wave: the 4 KiB of a tile's transpose
+// Extra (unused) LDS given to every workgroup of a launch with at least kAccThrottleTiles tiles: it
+// keeps a CU at 20 resident waves instead of 32, which measures 1-3 % faster on long vectors.  The
+// kernel is bound by how HBM copes with K thin read streams next to one wide write stream, and
+// fewer requests in flight serve it better; short vectors (one round of resident waves) want all
+// 32 slots instead.
+constexpr uint32_t kAccThrottleLdsBytes = 16384;
+constexpr uint64_t kAccThrottleTiles = 1u << 16;
 
-// 2-bit codes -> 2-bit two's complement multipliers, all 16 fields of a word at once:
-// 00 -> 00 (0), 01 -> 01 (+1), 10 -> 11 (-1), 11 -> 00 (0).  Per field (2 + b0 - b1) is 1..3,
-// so the subtraction never borrows across fields; xor 10 then gives the table above.
-__device__ __forceinline__ uint32_t codes_to_multipliers(uint32_t w)
+// Position in a wave's LDS area of 16-byte slot q (0..3) of row `row` (0..63; a row is the 16 sums
+// one lane owns).  Rows are 16 floats apart; the slot index is XOR-ed with bits of the row so that
+// both access patterns of the transpose are bank-conflict free for b128: a lane writing slot q of
+// its own row (8 consecutive lanes: rows r..r+7) and a lane reading slot lane&3 of row lane>>2 + 16j
+// (8 consecutive lanes: two rows, all four slots) each cover all 32 banks once.
+__device__ __forceinline__ int lds_slot(int row, int q) { return 16 * row + 4 * (q ^ ((row >> 1) & 3)); }
+
+// 2-bit codes -> 2 + b0 - b1 per field, all 16 fields of a word at once: 01 -> 11, 10 -> 01,
+// 00 and 11 -> 10.  Per field the value is 1..3, so the subtraction never borrows across fields.
+// Read as (sign, top exponent bit) of an IEEE half whose other bits are 0 these are -2, +2 and -0.
+__device__ __forceinline__ uint32_t codes_to_half_tops(uint32_t w)
 {
-    const uint32_t e = (w & 0x55555555u) | 0xAAAAAAAAu;
-    const uint32_t o = (w >> 1) & 0x55555555u;
-    return (e - o) ^ 0xAAAAAAAAu;
+    return ((w & 0x55555555u) | 0xAAAAAAAAu) - ((w >> 1) & 0x55555555u);
 }
 
 // acc[j] = ((start + d_0[j]) + d_1[j]) + ... strictly in payload order, start = accumulate ?
-// acc[j] : +0.0f.  With K payloads the sum costs K decodes and K adds per element, so the
-// layout is chosen for the arithmetic: a lane OWNS one code word of each payload (16 elements),
-// so a wave fetches a payload's 64 words with one coalesced 256 B load, every shift is an
+// acc[j] : +0.0f, for one tile of 1024 elements.  A lane OWNS one code word of each payload (16
+// elements): a wave fetches a payload's 64 words with one coalesced 256 B load, every shift is an
 // immediate, and nothing moves between lanes during the sum.  The 16 running sums of a lane are
-// 64 B apart in memory from its neighbour's, so the tile goes through LDS once on the way out
-// (and once on the way in when accumulating) to turn that into 1 KiB-contiguous stores.
+// 64 B apart in memory from its neighbour's, so the tile goes through LDS once on the way out (and
+// once on the way in when accumulating) to become 1 KiB-contiguous stores.
 //
-// FMA: when t is finite and not negative, (+t, -t, 0) is k * t with k in {+1, -1, 0} exactly and
-// fma(k, t, s) rounds s + k*t once, i.e. gives the same bits as s + decode: 3 VALU ops per
-// element and payload instead of 6 with compares and selects (which the K = 8 sum would be bound
-// by).  For any other t (negative, NaN, infinite: 0 * t would not be +0) the select form is used.
-template <int BLOCK, bool ALIGNED, bool NT, bool FMA>
-__global__ __launch_bounds__(BLOCK) void acc_flat_kernel(
-    float* acc, PayloadPtrs pl, int k_payloads, uint64_t n, uint64_t n_tiles, uint32_t has_tail,
-    uint32_t xs, float t, int accumulate)
+// K > 0: exactly K payloads (loop fully unrolled, no dead registers); K == 0: k_payloads of them,
+// at most NKLQ_MAX_PAYLOADS_PER_LAUNCH.
+//
+// MIX: for a finite t >= +0 whose half is exact, (+t, -t, +0) = h * th with th = -t/2 and h in
+// {-2, +2, -0} exactly, and fma(h, th, s) rounds s + h*th once: the same bits as s + decode.  h
+// is built as a half (the word's recoded field shifted to the top two bits of a 16-bit lane, two
+// elements per register) and consumed by the mixed-precision fma, which converts it for free:
+// one shift + one mask per TWO elements and one fma per element, against extract + convert + fma
+// per element for an integer multiplier, or two compares + two selects + add for the plain form.
+// Any other t (negative, NaN, infinite, below 2^-125) takes the plain form.
+template <int K, bool ALIGNED, bool MIX>
+__device__ __forceinline__ void acc_tile(float* o, const PayloadPtrs& pl, int k_payloads, uint64_t word0,
+                                         float t, float th, int accumulate, bool divide, float divisor,
+                                         float* my, int lane)
 {
-    constexpr int WPB = BLOCK / kWave;
-    __shared__ __attribute__((aligned(16))) float lds[WPB][kWave * kLdsLaneStride];
-    if (has_tail && blockIdx.x == gridDim.x - 1) {
-        // tail: fewer than 1024 elements, one per lane and round, bounds-checked
-        for (uint64_t e = n_tiles * kTile + threadIdx.x; e < n; e += BLOCK) {
-            const uint32_t sh = 2 * (uint32_t)(e & 15);
-            float s = accumulate ? acc[e] : 0.0f;
-            for (int p = 0; p < k_payloads; ++p) s = s + deq_code((pl.p[p][e >> 4] >> sh) & 3u, t);
-            acc[e] = s;
-        }
-        return;
-    }
-    const int lane = threadIdx.x & (kWave - 1);
-    const uint32_t w = threadIdx.x >> 6;
-    const uint64_t tile = chunk_of<1, BLOCK>(blockIdx.x, w, 0, xs);
-    if (tile >= n_tiles) return;
-    float* my = lds[w];
-    float* o = acc + tile * kTile;
-
+    constexpr int KMAX = K > 0 ? K : NKLQ_MAX_PAYLOADS_PER_LAUNCH;
     // every payload's word for this lane, all loads in flight together
-    uint32_t wd[NKLQ_MAX_PAYLOADS_PER_LAUNCH];
+    uint32_t wd[KMAX];
 #pragma unroll
-    for (int p = 0; p < NKLQ_MAX_PAYLOADS_PER_LAUNCH; ++p)
-        if (p < k_payloads) wd[p] = pl.p[p][tile * (kTile / 16) + lane];
+    for (int p = 0; p < KMAX; ++p)
+        if (K > 0 || p < k_payloads) wd[p] = pl.p[p][word0 + lane];
 
     float s[16];
     if (accumulate) {
         // coalesced read of the running sums, through LDS into the one-word-per-lane layout
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const f32x4 v = ld4<ALIGNED, NT>(o + j * 256 + lane * 4);
-            *reinterpret_cast<f32x4*>(my + lds_pos(j * 256 + lane * 4)) = v;
+            const f32x4 v = ld4<ALIGNED, true>(o + j * 256 + lane * 4);
+            *reinterpret_cast<f32x4*>(my + lds_slot(16 * j + (lane >> 2), lane & 3)) = v;
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-            const f32x4 v = *reinterpret_cast<const f32x4*>(my + kLdsLaneStride * lane + 4 * q);
+            const f32x4 v = *reinterpret_cast<const f32x4*>(my + lds_slot(lane, q));
             s[4 * q] = v.x; s[4 * q + 1] = v.y; s[4 * q + 2] = v.z; s[4 * q + 3] = v.w;
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -343,18 +342,26 @@ __global__ __launch_bounds__(BLOCK) void acc_flat_kernel(
     }
 
 #pragma unroll
-    for (int p = 0; p < NKLQ_MAX_PAYLOADS_PER_LAUNCH; ++p) {
-        if (p < k_payloads) {
-            if constexpr (FMA) {
-                const int m = (int)codes_to_multipliers(wd[p]);
+    for (int p = 0; p < KMAX; ++p) {
+        if (K > 0 || p < k_payloads) {
+            if constexpr (MIX) {
+                const uint32_t m = codes_to_half_tops(wd[p]);
 #pragma unroll
-                for (int i = 0; i < 16; ++i)
-                    s[i] = __builtin_fmaf((float)(int)__builtin_amdgcn_sbfe(m, 2 * i, 2), t, s[i]);
+                for (int i = 0; i < 8; ++i) {
+                    // elements i (low half) and i + 8 (high half) of the word
+                    const f16x2 h = __builtin_bit_cast(f16x2, (m << (14 - 2 * i)) & 0xC000C000u);
+                    s[i] = __builtin_fmaf((float)h.x, th, s[i]);
+                    s[i + 8] = __builtin_fmaf((float)h.y, th, s[i + 8]);
+                }
             } else {
 #pragma unroll
                 for (int i = 0; i < 16; ++i) s[i] = s[i] + deq_code((wd[p] >> (2 * i)) & 3u, t);
             }
         }
+    }
+    if (divide) {  // IEEE division, correctly rounded (not a reciprocal)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[i] = s[i] / divisor;
     }
 
     // one-word-per-lane layout -> LDS -> 1 KiB-contiguous stores
@@ -362,16 +369,65 @@ __global__ __launch_bounds__(BLOCK) void acc_flat_kernel(
     for (int q = 0; q < 4; ++q) {
         f32x4 v;
         v.x = s[4 * q]; v.y = s[4 * q + 1]; v.z = s[4 * q + 2]; v.w = s[4 * q + 3];
-        *reinterpret_cast<f32x4*>(my + kLdsLaneStride * lane + 4 * q) = v;
+        *reinterpret_cast<f32x4*>(my + lds_slot(lane, q)) = v;
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        const f32x4 v = *reinterpret_cast<const f32x4*>(my + lds_pos(j * 256 + lane * 4));
-        st4<ALIGNED, NT>(o + j * 256 + lane * 4, v);
+        const f32x4 v = *reinterpret_cast<const f32x4*>(my + lds_slot(16 * j + (lane >> 2), lane & 3));
+        st4<ALIGNED, true>(o + j * 256 + lane * 4, v);
     }
+}
+
+// Fewer than 1024 elements [e0, n) of one vector, bounds-checked: a lane takes elements first,
+// first + step, ... four at a time, so that four loads per payload are in flight instead of one.
+__device__ __forceinline__ void acc_partial_tile(float* acc, const PayloadPtrs& pl, int k_payloads,
+                                                 uint64_t word_offset, uint64_t e0, uint64_t n, float t,
+                                                 int accumulate, bool divide, float divisor, int first,
+                                                 int step)
+{
+    for (uint64_t base = e0 + first; base < n; base += 4 * (uint64_t)step) {
+        uint64_t e[4];
+        float s[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            e[r] = base + (uint64_t)r * step;
+            s[r] = (accumulate && e[r] < n) ? acc[e[r]] : 0.0f;
+        }
+#pragma unroll 2
+        for (int p = 0; p < k_payloads; ++p) {
+            const uint32_t* words = pl.p[p] + word_offset;
+            uint32_t wd[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) wd[r] = e[r] < n ? words[e[r] >> 4] : 0u;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) s[r] = s[r] + deq_code((wd[r] >> (2 * (uint32_t)(e[r] & 15))) & 3u, t);
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            if (e[r] < n) acc[e[r]] = divide ? s[r] / divisor : s[r];
+    }
+}
+
+template <int K, bool ALIGNED, bool MIX>
+__global__ __launch_bounds__(kAccBlock) void acc_flat_kernel(
+    float* acc, PayloadPtrs pl, int k_payloads, uint64_t n, uint64_t n_tiles, uint32_t has_tail,
+    uint32_t xs, float t, float th, int accumulate)
+{
+    __shared__ __attribute__((aligned(16))) float lds[kAccBlock / kWave][kAccLdsPerWave];
+    if (has_tail && blockIdx.x == gridDim.x - 1) {
+        acc_partial_tile(acc, pl, k_payloads, 0, n_tiles * kTile, n, t, accumulate, false, 1.0f,
+                         threadIdx.x, kAccBlock);
+        return;
+    }
+    const int lane = threadIdx.x & (kWave - 1);
+    const uint32_t w = threadIdx.x >> 6;
+    const uint64_t tile = chunk_of<1, kAccBlock>(blockIdx.x, w, 0, xs);
+    if (tile >= n_tiles) return;
+    acc_tile<K, ALIGNED, MIX>(acc + tile * kTile, pl, k_payloads, tile * (kTile / 16), t, th, accumulate,
+                              false, 1.0f, lds[w], lane);
 }
 
 // ---------------------------------------------------------------- matrix (n, k) kernels
@@ -634,93 +690,29 @@ struct AccSegments {
     int count;
 };
 
-template <bool ALIGNED, bool NT, bool FMA>
-__global__ __launch_bounds__(256) void acc_multi_kernel(AccSegments seg, PayloadPtrs pl, int k_payloads,
-                                                        uint32_t xs, float t, int accumulate,
-                                                        float divisor)
+template <int K, bool ALIGNED, bool MIX>
+__global__ __launch_bounds__(kAccBlock) void acc_multi_kernel(AccSegments seg, PayloadPtrs pl, int k_payloads,
+                                                              uint32_t xs, float t, float th, int accumulate,
+                                                              float divisor)
 {
-    const bool divide = divisor != 1.0f;  // IEEE division, correctly rounded (not a reciprocal)
-    __shared__ __attribute__((aligned(16))) float lds[4][kWave * kLdsLaneStride];
+    const bool divide = divisor != 1.0f;
+    __shared__ __attribute__((aligned(16))) float lds[kAccBlock / kWave][kAccLdsPerWave];
     const int lane = threadIdx.x & (kWave - 1);
     const uint32_t w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const uint64_t q64 = chunk_of<1, 256>(blockIdx.x, w, 0, xs);
+    const uint64_t q64 = chunk_of<1, kAccBlock>(blockIdx.x, w, 0, xs);
     if (q64 >= seg.first[seg.count]) return;
     const uint32_t q = (uint32_t)q64;
     const int sidx = find_segment(seg.first, seg.count, q);
     const uint64_t n = seg.n[sidx];
     const uint64_t e0 = (uint64_t)(q - seg.first[sidx]) * kTile;
-    float* o = seg.acc[sidx] + e0;
-    const uint64_t w0 = seg.word_offset[sidx] + (e0 >> 4);
     if (e0 + kTile > n) {
-        // last, partial tile of the vector: one element per lane and round, bounds-checked
-        for (uint64_t e = e0 + lane; e < n; e += kWave) {
-            const uint32_t sh = 2 * (uint32_t)(e & 15);
-            float s = accumulate ? seg.acc[sidx][e] : 0.0f;
-            for (int p = 0; p < k_payloads; ++p)
-                s = s + deq_code((pl.p[p][seg.word_offset[sidx] + (e >> 4)] >> sh) & 3u, t);
-            seg.acc[sidx][e] = divide ? s / divisor : s;
-        }
+        // last, partial tile of the vector
+        acc_partial_tile(seg.acc[sidx], pl, k_payloads, seg.word_offset[sidx], e0, n, t, accumulate,
+                         divide, divisor, lane, kWave);
         return;
     }
-    float* my = lds[w];
-    uint32_t wd[NKLQ_MAX_PAYLOADS_PER_LAUNCH];
-#pragma unroll
-    for (int p = 0; p < NKLQ_MAX_PAYLOADS_PER_LAUNCH; ++p)
-        if (p < k_payloads) wd[p] = pl.p[p][w0 + lane];
-    float s[16];
-    if (accumulate) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const f32x4 v = ld4<ALIGNED, NT>(o + j * 256 + lane * 4);
-            *reinterpret_cast<f32x4*>(my + lds_pos(j * 256 + lane * 4)) = v;
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-#pragma unroll
-        for (int qd = 0; qd < 4; ++qd) {
-            const f32x4 v = *reinterpret_cast<const f32x4*>(my + kLdsLaneStride * lane + 4 * qd);
-            s[4 * qd] = v.x; s[4 * qd + 1] = v.y; s[4 * qd + 2] = v.z; s[4 * qd + 3] = v.w;
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    } else {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) s[i] = 0.0f;
-    }
-#pragma unroll
-    for (int p = 0; p < NKLQ_MAX_PAYLOADS_PER_LAUNCH; ++p) {
-        if (p < k_payloads) {
-            if constexpr (FMA) {
-                const int m = (int)codes_to_multipliers(wd[p]);
-#pragma unroll
-                for (int i = 0; i < 16; ++i)
-                    s[i] = __builtin_fmaf((float)(int)__builtin_amdgcn_sbfe(m, 2 * i, 2), t, s[i]);
-            } else {
-#pragma unroll
-                for (int i = 0; i < 16; ++i) s[i] = s[i] + deq_code((wd[p] >> (2 * i)) & 3u, t);
-            }
-        }
-    }
-    if (divide) {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) s[i] = s[i] / divisor;
-    }
-#pragma unroll
-    for (int qd = 0; qd < 4; ++qd) {
-        f32x4 v;
-        v.x = s[4 * qd]; v.y = s[4 * qd + 1]; v.z = s[4 * qd + 2]; v.w = s[4 * qd + 3];
-        *reinterpret_cast<f32x4*>(my + kLdsLaneStride * lane + 4 * qd) = v;
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const f32x4 v = *reinterpret_cast<const f32x4*>(my + lds_pos(j * 256 + lane * 4));
-        st4<ALIGNED, NT>(o + j * 256 + lane * 4, v);
-    }
+    acc_tile<K, ALIGNED, MIX>(seg.acc[sidx] + e0, pl, k_payloads, seg.word_offset[sidx] + (e0 >> 4), t, th,
+                              accumulate, divide, divisor, lds[w], lane);
 }
 
 // ---------------------------------------------------------------- copy (measurement aid)
@@ -755,7 +747,8 @@ int g_chunks_per_wave = 1;  // 1, 2 or 4
 int g_block = 256;          // 64, 128, 256, 512 or 1024 threads
 int g_nontemporal = 1;
 int g_xcd_shift = 2;        // quantize/copy: chunks interleaved over 2^g_xcd_shift workgroups
-int g_xcd_shift_decode = 0; // the same for dequantize and accumulate (write-dominated: contiguous wins)
+int g_xcd_shift_decode = 0; // the same for dequantize (write-dominated: contiguous wins)
+int g_xcd_shift_acc = 3;    // the same for the sum over payloads (tiles of 1024 elements, dealt over all 8 XCDs)
 
 int compute_units()
 {
@@ -846,37 +839,55 @@ int launch_deq_flat(float* out, const uint32_t* c, uint64_t n, float t, hipStrea
     return launch_status();
 }
 
-// The accumulate kernel works on tiles of 1024 elements, one per wave, 256-thread workgroups.
+// The fast form of the sum needs 0 * t = +0, an exact t/2 and exact products: finite t >= +0 with
+// a biased exponent of at least 2 (or t = +0).
+inline bool mix_ok(float t)
+{
+    const uint32_t b = __builtin_bit_cast(uint32_t, t);
+    const uint32_t ex = (b >> 23) & 0xFFu;
+    return (b >> 31) == 0 && ex != 0xFFu && (ex >= 2 || b == 0);
+}
+
+// Instantiates BODY(K, AL, MIX) for the payload count k: K = k up to 8 (unrolled), else K = 0 (the
+// runtime-count form); the plain (non-MIX) form only exists with K = 0.
+#define NKLQ_ACC_DISPATCH(BODY, k, al, mix)                                          \
+    do {                                                                             \
+        if (!(mix)) {                                                                \
+            if (al) BODY(0, true, false); else BODY(0, false, false);                \
+        } else {                                                                     \
+            switch ((k) <= 8 ? (k) : 0) {                                            \
+                case 1: if (al) BODY(1, true, true); else BODY(1, false, true); break; \
+                case 2: if (al) BODY(2, true, true); else BODY(2, false, true); break; \
+                case 3: if (al) BODY(3, true, true); else BODY(3, false, true); break; \
+                case 4: if (al) BODY(4, true, true); else BODY(4, false, true); break; \
+                case 5: if (al) BODY(5, true, true); else BODY(5, false, true); break; \
+                case 6: if (al) BODY(6, true, true); else BODY(6, false, true); break; \
+                case 7: if (al) BODY(7, true, true); else BODY(7, false, true); break; \
+                case 8: if (al) BODY(8, true, true); else BODY(8, false, true); break; \
+                default: if (al) BODY(0, true, true); else BODY(0, false, true); break; \
+            }                                                                        \
+        }                                                                            \
+    } while (0)
+
+// The accumulate kernels work on tiles of 1024 elements, one per wave, 256-thread workgroups.
 int launch_acc_flat(float* acc, const PayloadPtrs& pl, int k, uint64_t n, float t, int accumulate,
                     hipStream_t s)
 {
-    constexpr int BLOCK = 256;
-    const uint32_t xs = (uint32_t)g_xcd_shift_decode;
     const uint64_t n_tiles = n / kTile;
     const uint32_t has_tail = (n_tiles * kTile < n) ? 1u : 0u;
-    const uint64_t per_group = (uint64_t)(BLOCK / kWave) << xs;
+    const uint32_t xs = (uint32_t)g_xcd_shift_acc;
+    const uint64_t per_group = (uint64_t)(kAccBlock / kWave) << xs;
     const uint64_t work = ((n_tiles + per_group - 1) / per_group) << xs;
     if (work + has_tail > 0x7FFFFFFFull) return NKLQ_ERANGE;
     const uint32_t blocks = (uint32_t)work + has_tail;
     const bool al = aligned16(acc);
-    const bool nt = g_nontemporal != 0;
-    // fma(k, t, s) reproduces s + decode only when 0 * t is +0 and k * t is exact: finite t >= +0
-    const uint32_t tbits = __builtin_bit_cast(uint32_t, t);
-    const bool fma_ok = (tbits >> 31) == 0 && (tbits & 0x7F800000u) != 0x7F800000u;
-#define NKLQ_ACC(AL, NT, FMA)                                                                     \
-    hipLaunchKernelGGL((acc_flat_kernel<BLOCK, AL, NT, FMA>), dim3(blocks), dim3(BLOCK), 0, s, acc, \
-                       pl, k, n, n_tiles, has_tail, xs, t, accumulate)
-    const int sel = (al ? 4 : 0) | (nt ? 2 : 0) | (fma_ok ? 1 : 0);
-    switch (sel) {
-        case 7: NKLQ_ACC(true, true, true); break;
-        case 6: NKLQ_ACC(true, true, false); break;
-        case 5: NKLQ_ACC(true, false, true); break;
-        case 4: NKLQ_ACC(true, false, false); break;
-        case 3: NKLQ_ACC(false, true, true); break;
-        case 2: NKLQ_ACC(false, true, false); break;
-        case 1: NKLQ_ACC(false, false, true); break;
-        default: NKLQ_ACC(false, false, false); break;
-    }
+    const bool mix = mix_ok(t);
+    const float th = -0.5f * t;
+    const uint32_t pad = n_tiles >= kAccThrottleTiles ? kAccThrottleLdsBytes : 0u;
+#define NKLQ_ACC(K, AL, MIX)                                                                        \
+    hipLaunchKernelGGL((acc_flat_kernel<K, AL, MIX>), dim3(blocks), dim3(kAccBlock), pad, s, acc, pl, k, n, \
+                       n_tiles, has_tail, xs, t, th, accumulate)
+    NKLQ_ACC_DISPATCH(NKLQ_ACC, k, al, mix);
 #undef NKLQ_ACC
     return launch_status();
 }
@@ -975,25 +986,16 @@ int launch_acc_multi(const AccSegments& seg, const PayloadPtrs& pl, int k, bool 
                      int accumulate, float divisor, hipStream_t s)
 {
     uint32_t blocks;
-    const uint32_t xs = (uint32_t)g_xcd_shift_decode;
+    const uint32_t xs = (uint32_t)g_xcd_shift_acc;
     if (!multi_grid(seg.first[seg.count], xs, &blocks)) return NKLQ_ERANGE;
     if (blocks == 0) return NKLQ_OK;
-    const bool nt = g_nontemporal != 0;
-    const uint32_t tbits = __builtin_bit_cast(uint32_t, t);
-    const bool fma_ok = (tbits >> 31) == 0 && (tbits & 0x7F800000u) != 0x7F800000u;
-#define NKLQ_AM(AL, NT, FMA)                                                                      \
-    hipLaunchKernelGGL((acc_multi_kernel<AL, NT, FMA>), dim3(blocks), dim3(256), 0, s, seg, pl, k, xs, \
-                       t, accumulate, divisor)
-    switch ((al ? 4 : 0) | (nt ? 2 : 0) | (fma_ok ? 1 : 0)) {
-        case 7: NKLQ_AM(true, true, true); break;
-        case 6: NKLQ_AM(true, true, false); break;
-        case 5: NKLQ_AM(true, false, true); break;
-        case 4: NKLQ_AM(true, false, false); break;
-        case 3: NKLQ_AM(false, true, true); break;
-        case 2: NKLQ_AM(false, true, false); break;
-        case 1: NKLQ_AM(false, false, true); break;
-        default: NKLQ_AM(false, false, false); break;
-    }
+    const bool mix = mix_ok(t);
+    const float th = -0.5f * t;
+    const uint32_t pad = seg.first[seg.count] >= kAccThrottleTiles ? kAccThrottleLdsBytes : 0u;
+#define NKLQ_AM(K, AL, MIX)                                                                           \
+    hipLaunchKernelGGL((acc_multi_kernel<K, AL, MIX>), dim3(blocks), dim3(kAccBlock), pad, s, seg, pl, k, xs, \
+                       t, th, accumulate, divisor)
+    NKLQ_ACC_DISPATCH(NKLQ_AM, k, al, mix);
 #undef NKLQ_AM
     return launch_status();
 }
@@ -1050,6 +1052,7 @@ int nklq_tune(int which, int value)
         case NKLQ_TUNE_NONTEMPORAL: slot = &g_nontemporal; break;
         case NKLQ_TUNE_XCD_INTERLEAVE_LOG2: slot = &g_xcd_shift; break;
         case NKLQ_TUNE_XCD_INTERLEAVE_LOG2_DECODE: slot = &g_xcd_shift_decode; break;
+        case NKLQ_TUNE_XCD_INTERLEAVE_LOG2_ACCUMULATE: slot = &g_xcd_shift_acc; break;
         default: return NKLQ_ERANGE;
     }
     const int prev = *slot;

@@ -21,11 +21,11 @@ FLAT_SIZES = list(range(1, 50)) + [63, 64, 65, 255, 256, 257, 1023, 1024, 1025, 
 def _knobs():
     """Launch geometries to run every flat test under; results must not depend on them."""
     default = tuple(_lib.tune(i) for i in range(_lib.N_TUNE))
-    return [default, (1, 64, 1, 3, 1), (2, 128, 0, 0, 2), (4, 256, 1, 3, 3), (4, 1024, 0, 5, 6),
-            (2, 512, 1, 6, 0), (1, 1024, 1, 1, 4)]
+    return [default, (1, 64, 1, 3, 1, 0), (2, 128, 0, 0, 2, 1), (4, 256, 1, 3, 3, 2), (4, 1024, 0, 5, 6, 4),
+            (2, 512, 1, 6, 0, 6), (1, 1024, 1, 1, 4, 5)]
 
 
-@pytest.fixture(params=_knobs(), ids=lambda k: f"u{k[0]}-wg{k[1]}-nt{k[2]}-x{k[3]}-xd{k[4]}")
+@pytest.fixture(params=_knobs(), ids=lambda k: f"u{k[0]}-wg{k[1]}-nt{k[2]}-x{k[3]}-xd{k[4]}-xa{k[5]}")
 def knobs(request):
     old = [_lib.tune(i) for i in range(_lib.N_TUNE)]
     for i, v in enumerate(request.param):
