@@ -131,6 +131,29 @@ __device__ __forceinline__ void st4(float* p, f32x4 v)
     }
 }
 
+// Store of a lane's 16 bytes inside a wave's 1 KiB piece that may start anywhere: the first and
+// the last 128-byte line of a piece that starts off a line are shared with the neighbouring pieces
+// (other waves).  A streaming (non-temporal) store of part of a line goes to memory as a
+// partial-line write; that is harmless when the cut falls on a 32-byte sector, but a cut inside a
+// sector makes memory read, merge and write the sector.  In that case the lanes on those two lines
+// store with the ordinary policy instead, so that the halves meet in L2 (the neighbouring piece is
+// written from the same XCD, and the line is already there from the residual's load) and leave it
+// as whole sectors.
+template <bool ALIGNED, bool NT>
+__device__ __forceinline__ void st4_piece(float* p, f32x4 v, int lane)
+{
+    if constexpr (NT) {
+        const uintptr_t a = reinterpret_cast<uintptr_t>(p);
+        const uintptr_t piece = a - (uintptr_t)lane * 16;  // lane 0's address
+        const bool cut_in_sector = (piece & 31u) != 0;
+        const bool edge = cut_in_sector && ((a >> 7) == (piece >> 7) || ((a + 15) >> 7) == ((piece + 1023) >> 7));
+        if (edge) st4<ALIGNED, false>(p, v);
+        else st4<ALIGNED, true>(p, v);
+    } else {
+        st4<ALIGNED, false>(p, v);
+    }
+}
+
 // ---------------------------------------------------------------- chunk -> workgroup map
 
 // Workgroups are handed to the XCDs round-robin by workgroup id.  With
@@ -442,7 +465,22 @@ __global__ __launch_bounds__(kAccBlock) void acc_flat_kernel(
 // aligned) rows start at any element: ALIGNED = false issues the same loads with dword
 // alignment, and the last 1-3 columns of a row are moved one by one.
 constexpr int kRowsBlock = 16 * kWave;  // 1024 threads
-constexpr uint64_t kNarrowColumns = 64; // below this many columns the one-lane-per-word kernels run
+
+// Workgroup -> tile (word row x, column tile T).  Workgroups go to the 8 XCDs round-robin by id; the
+// tiles of one word row are given to ONE XCD, in column order, and 8 neighbouring word rows run
+// side by side on the 8 XCDs.  When rows do not start on cache-line boundaries (k not a multiple
+// of 32) neighbouring tiles of a row share a line at their common edge: written from one XCD the
+// two halves merge in that XCD's L2 into a full-line write, written from two XCDs they reach memory
+// as two partial-line writes.  Returns false for the padding workgroups of the last group of rows.
+__device__ __forceinline__ bool rows_tile_of(uint32_t b, uint32_t col_tiles, uint64_t m, uint64_t* x,
+                                             uint32_t* T)
+{
+    const uint32_t e = b & 7u;
+    const uint32_t j = b >> 3;
+    *x = (uint64_t)(j / col_tiles) * 8 + e;
+    *T = j % col_tiles;
+    return *x < m;
+}
 
 template <bool ADD, bool NT, bool ALIGNED>
 __global__ __launch_bounds__(kRowsBlock) void quant_2d_rows_kernel(
@@ -452,8 +490,10 @@ __global__ __launch_bounds__(kRowsBlock) void quant_2d_rows_kernel(
     __shared__ uint32_t words[256];
     const int lane = threadIdx.x & (kWave - 1);
     const uint32_t i = threadIdx.x >> 6;  // row inside the tile = code position inside the word
-    const uint64_t x = blockIdx.x / col_tiles;
-    const uint64_t y0 = (uint64_t)(blockIdx.x % col_tiles) * 256;
+    uint64_t x;
+    uint32_t T;
+    if (!rows_tile_of(blockIdx.x, col_tiles, (n + 15) / 16, &x, &T)) return;
+    const uint64_t y0 = (uint64_t)T * 256;
     const uint64_t y = y0 + (uint64_t)lane * 4;
     const uint64_t row = x * 16 + i;
     // columns this lane owns: 4, or fewer at the right edge, or none
@@ -492,7 +532,7 @@ __global__ __launch_bounds__(kRowsBlock) void quant_2d_rows_kernel(
         if (cnt == 4) {
             f32x4 vo;
             vo.x = o[0]; vo.y = o[1]; vo.z = o[2]; vo.w = o[3];
-            st4<ALIGNED, NT>(rout + off, vo);
+            st4_piece<ALIGNED, NT>(rout + off, vo, lane);
         } else {
 #pragma unroll
             for (int j = 0; j < 3; ++j)
@@ -509,29 +549,37 @@ __global__ __launch_bounds__(kRowsBlock) void quant_2d_rows_kernel(
         c[x * k + y0 + threadIdx.x] = words[64 * (threadIdx.x & 3) + (threadIdx.x >> 2)];
 }
 
-template <bool NT, bool ALIGNED>
+// Decode of a tile.  SHIFT = false: every row starts on a 128-byte line (k a multiple of 32, base
+// on a line) and wave i writes columns [256 T, 256 T + 256) of its row.  SHIFT = true: each row's
+// window is moved left by the s = 0..31 elements its start lies past a line, so that a wave still
+// writes whole, aligned lines: columns [256 T - s, 256 T + 256 - s), clipped to the row (one more
+// column tile covers the rows' ends).  Nothing is shared between rows here, so the windows of the
+// 16 rows need not coincide; only the first and last line of a row are partial.  All 16 waves
+// read the tile's words (cache hits after the first).
+template <bool NT, bool SHIFT>
 __global__ __launch_bounds__(kRowsBlock) void deq_2d_rows_kernel(
     float* out, const uint32_t* __restrict__ c, uint64_t n, uint64_t k, uint32_t col_tiles, float t)
 {
     const int lane = threadIdx.x & (kWave - 1);
     const uint32_t i = threadIdx.x >> 6;
-    const uint64_t x = blockIdx.x / col_tiles;
-    const uint64_t y = (uint64_t)(blockIdx.x % col_tiles) * 256 + (uint64_t)lane * 4;
+    uint64_t x;
+    uint32_t T;
+    if (!rows_tile_of(blockIdx.x, col_tiles, (n + 15) / 16, &x, &T)) return;
     const uint64_t row = x * 16 + i;
-    if (row >= n || y >= k) return;
-    // with ALIGNED, k is a multiple of 4 and every lane inside the matrix owns 4 columns
-    const int cnt = ALIGNED ? 4 : ((k - y < 4) ? (int)(k - y) : 4);
+    if (row >= n) return;
+    float* orow = out + row * k;
+    const int64_t s = SHIFT ? (int64_t)((reinterpret_cast<uintptr_t>(orow) >> 2) & 31u) : 0;
+    const int64_t y = (int64_t)T * 256 - s + lane * 4;  // first of this lane's 4 columns
+    if (y >= (int64_t)k || y + 4 <= 0) return;
     const uint32_t sh = 2 * i;
-    const uint32_t* cw = c + x * k + y;
-    float* o = out + row * k + y;
-    // all 16 waves read the tile's 1 KiB of words (cache hits after the first)
-    if (cnt == 4) {
+    const uint32_t* cw = c + x * k;
+    if (y >= 0 && y + 4 <= (int64_t)k) {
         uint32_t w0, w1, w2, w3;
-        if constexpr (ALIGNED) {
-            const u32x4 w = *reinterpret_cast<const u32x4*>(cw);
+        if constexpr (SHIFT) {
+            const u32x4_a4 w = *reinterpret_cast<const u32x4_a4*>(cw + y);
             w0 = w.x; w1 = w.y; w2 = w.z; w3 = w.w;
         } else {
-            const u32x4_a4 w = *reinterpret_cast<const u32x4_a4*>(cw);
+            const u32x4 w = *reinterpret_cast<const u32x4*>(cw + y);
             w0 = w.x; w1 = w.y; w2 = w.z; w3 = w.w;
         }
         f32x4 v;
@@ -539,67 +587,157 @@ __global__ __launch_bounds__(kRowsBlock) void deq_2d_rows_kernel(
         v.y = deq_code((w1 >> sh) & 3u, t);
         v.z = deq_code((w2 >> sh) & 3u, t);
         v.w = deq_code((w3 >> sh) & 3u, t);
-        st4<ALIGNED, NT>(o, v);
+        st4<true, NT>(orow + y, v);  // 16-byte aligned in both forms
     } else {
-        for (int j = 0; j < cnt; ++j) o[j] = deq_code((cw[j] >> sh) & 3u, t);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (y + j >= 0 && y + j < (int64_t)k) orow[y + j] = deq_code((cw[y + j] >> sh) & 3u, t);
     }
 }
 
-constexpr int kBlock2D = 256;  // workgroup size of the narrow-matrix kernels
+// ---- matrices of up to kBandsMaxColumns columns
+//
+// The 16 rows behind one row of code words ("a band") are 16 k CONTIGUOUS floats in memory and
+// give k contiguous words.  With few columns a 256-column tile would leave most lanes idle, and
+// walking down a column touches one float per row; instead a workgroup takes whole bands as a
+// flat stream: `bands_per_wg` bands when a band is short (so that the range is 2048-4096
+// elements), one band otherwise.  The range is read and written 16 bytes per lane like a flat vector
+// (quads laid out from a 16-byte boundary of the residual, so only the first and last quad of a range
+// can be partial and go element by element), each element finds its (row, column) by one
+// multiply-high with a precomputed reciprocal of k, and its code is OR-ed into the band's words in
+// LDS; after a barrier the words are stored, contiguous.
+constexpr int kBandsBlock = 256;
+constexpr uint64_t kBandsMaxColumns = 384;  // LDS words per workgroup; wider matrices take the row tiles (measured crossover: 300-500 columns)
+constexpr uint64_t kBandsRangeQuant = 2048;   // elements per workgroup when bands are short: quantize
+constexpr uint64_t kBandsRangeDecode = 4096;  // and decode (measured)
 
-// Narrow matrices (k < 64 columns): a 256-column tile would leave most lanes idle, so one lane
-// takes one word and lanes walk along the flattened (x, y) index.
-template <bool ADD>
-__global__ __launch_bounds__(kBlock2D) void quant_2d_kernel(
-    const float* g, const float* rin, float* rout, uint32_t* __restrict__ c, uint64_t n,
-    uint64_t k, uint64_t items, float t)
+// (row within the workgroup's range, column) of local element index li; inv = floor(2^32 / k) + 1,
+// exact for li * k < 2^32 (li < 16384, k <= 1024 here).
+__device__ __forceinline__ void band_row_col(uint32_t li, uint32_t k, uint32_t inv, uint32_t* row, uint32_t* col)
 {
-    for (uint64_t it = (uint64_t)blockIdx.x * kBlock2D + threadIdx.x; it < items;
-         it += (uint64_t)gridDim.x * kBlock2D) {
-        const uint64_t x = it / k;
-        const uint64_t y = it - x * k;
-        uint32_t word = 0;
+    const uint32_t q = __umulhi(li, inv);
+    *row = q;
+    *col = li - q * k;
+}
+
+template <bool ADD, bool NT, bool ALIGNED>
+__global__ __launch_bounds__(kBandsBlock) void quant_bands_kernel(
+    const float* g, const float* rin, float* rout, uint32_t* __restrict__ c, uint64_t n, uint32_t k,
+    uint32_t bands_per_wg, uint32_t inv, float t)
+{
+    __shared__ uint32_t words[kBandsMaxColumns];
+    const uint64_t m = (n + 15) / 16;
+    const uint64_t x0 = (uint64_t)blockIdx.x * bands_per_wg;
+    const uint64_t x1 = (x0 + bands_per_wg < m) ? x0 + bands_per_wg : m;
+    const uint64_t e0 = x0 * 16 * k;
+    const uint64_t e1 = (x1 * 16 < n ? x1 * 16 : n) * k;
+    const uint32_t n_words = (uint32_t)(x1 - x0) * k;
+    const uint32_t len = (uint32_t)(e1 - e0);
+    for (uint32_t w = threadIdx.x; w < n_words; w += kBandsBlock) words[w] = 0;
+    __syncthreads();
+    // quads start `a` elements before the range, on a 16-byte boundary of rout
+    const uint32_t a = (uint32_t)((reinterpret_cast<uintptr_t>(rout + e0) >> 2) & 3u);
+    const float* gq = g + e0;
+    const float* rq = rin + e0;
+    float* oq = rout + e0;
+    // local index of a quad's first element, relative to e0: -a + 4 * quad (negative only for quad 0)
+    constexpr int U = 4;  // quads per lane whose loads are issued together
+    for (int32_t base = -(int32_t)a + 4 * (int32_t)threadIdx.x; base < (int32_t)len; base += U * 4 * kBandsBlock) {
+        f32x4 va[U], vr[U];
 #pragma unroll
-        for (int half = 0; half < 2; ++half) {
-            float a[8];
-            float r[8];
+        for (int u = 0; u < U; ++u) {
+            const int32_t li = base + u * 4 * kBandsBlock;
+            if (li >= 0 && li + 4 <= (int32_t)len) {
+                va[u] = ld4<ALIGNED, NT>(gq + li);
+                if constexpr (ADD) vr[u] = ld4<ALIGNED, NT>(rq + li);
+            } else {
+                float xa[4] = {0.0f, 0.0f, 0.0f, 0.0f}, xr[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const uint64_t xm = x * 16 + half * 8 + i;
-                if (xm < n) {
-                    a[i] = g[xm * k + y];
-                    if constexpr (ADD) r[i] = rin[xm * k + y];
+                for (int j = 0; j < 4; ++j) {
+                    if (li + j >= 0 && li + j < (int32_t)len) {
+                        xa[j] = gq[li + j];
+                        if constexpr (ADD) xr[j] = rq[li + j];
+                    }
                 }
+                va[u].x = xa[0]; va[u].y = xa[1]; va[u].z = xa[2]; va[u].w = xa[3];
+                if constexpr (ADD) { vr[u].x = xr[0]; vr[u].y = xr[1]; vr[u].z = xr[2]; vr[u].w = xr[3]; }
             }
+        }
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const uint64_t xm = x * 16 + half * 8 + i;
-                if (xm < n) {
-                    float val = a[i];
-                    if constexpr (ADD) val = val + r[i];
-                    float o;
-                    word |= quant_one(val, t, o) << (2 * (half * 8 + i));
-                    rout[xm * k + y] = o;
+        for (int u = 0; u < U; ++u) {
+            const int32_t li = base + u * 4 * kBandsBlock;
+            if (li >= (int32_t)len) break;
+            f32x4 v = va[u];
+            if constexpr (ADD) v = v + vr[u];
+            float in[4] = {v.x, v.y, v.z, v.w};
+            float o[4];
+            uint32_t code[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) code[j] = quant_one(in[j], t, o[j]);
+            const bool full = li >= 0 && li + 4 <= (int32_t)len;
+            if (full) {
+                f32x4 vo;
+                vo.x = o[0]; vo.y = o[1]; vo.z = o[2]; vo.w = o[3];
+                st4<true, NT>(oq + li, vo);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    if (li + j >= 0 && li + j < (int32_t)len) oq[li + j] = o[j];
+            }
+            uint32_t row, col;
+            band_row_col((uint32_t)(li < 0 ? 0 : li), k, inv, &row, &col);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if (li + j >= 0 && li + j < (int32_t)len) {
+                    // word of (row, col): band row / 16 of this range, bits of row % 16
+                    if (code[j]) atomicOr(&words[(row >> 4) * k + col], code[j] << (2 * (row & 15u)));
+                    if (++col == k) { col = 0; ++row; }
                 }
             }
         }
-        c[x * k + y] = word;
     }
+    __syncthreads();
+    uint32_t* cq = c + x0 * k;
+    for (uint32_t w = threadIdx.x; w < n_words; w += kBandsBlock) cq[w] = words[w];
 }
 
-__global__ __launch_bounds__(kBlock2D) void deq_2d_kernel(float* out, const uint32_t* __restrict__ c,
-                                                           uint64_t n, uint64_t k, uint64_t items,
-                                                           float t)
+template <bool NT>
+__global__ __launch_bounds__(kBandsBlock) void deq_bands_kernel(
+    float* out, const uint32_t* __restrict__ c, uint64_t n, uint32_t k, uint32_t bands_per_wg, uint32_t inv,
+    float t)
 {
-    for (uint64_t it = (uint64_t)blockIdx.x * kBlock2D + threadIdx.x; it < items;
-         it += (uint64_t)gridDim.x * kBlock2D) {
-        const uint64_t x = it / k;
-        const uint64_t y = it - x * k;
-        const uint32_t word = c[x * k + y];
+    __shared__ uint32_t words[kBandsMaxColumns];
+    const uint64_t m = (n + 15) / 16;
+    const uint64_t x0 = (uint64_t)blockIdx.x * bands_per_wg;
+    const uint64_t x1 = (x0 + bands_per_wg < m) ? x0 + bands_per_wg : m;
+    const uint64_t e0 = x0 * 16 * k;
+    const uint64_t e1 = (x1 * 16 < n ? x1 * 16 : n) * k;
+    const uint32_t n_words = (uint32_t)(x1 - x0) * k;
+    const uint32_t len = (uint32_t)(e1 - e0);
+    const uint32_t* cq = c + x0 * k;
+    for (uint32_t w = threadIdx.x; w < n_words; w += kBandsBlock) words[w] = cq[w];
+    __syncthreads();
+    const uint32_t a = (uint32_t)((reinterpret_cast<uintptr_t>(out + e0) >> 2) & 3u);
+    float* oq = out + e0;
+    for (int32_t li = -(int32_t)a + 4 * (int32_t)threadIdx.x; li < (int32_t)len; li += 4 * kBandsBlock) {
+        uint32_t row, col;
+        band_row_col((uint32_t)(li < 0 ? 0 : li), k, inv, &row, &col);
+        float o[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const uint64_t xm = x * 16 + i;
-            if (xm < n) out[xm * k + y] = deq_code((word >> (2 * i)) & 3u, t);
+        for (int j = 0; j < 4; ++j) {
+            if (li + j >= 0 && li + j < (int32_t)len) {
+                o[j] = deq_code((words[(row >> 4) * k + col] >> (2 * (row & 15u))) & 3u, t);
+                if (++col == k) { col = 0; ++row; }
+            }
+        }
+        if (li >= 0 && li + 4 <= (int32_t)len) {
+            f32x4 vo;
+            vo.x = o[0]; vo.y = o[1]; vo.z = o[2]; vo.w = o[3];
+            st4<true, NT>(oq + li, vo);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (li + j >= 0 && li + j < (int32_t)len) oq[li + j] = o[j];
         }
     }
 }
@@ -1000,12 +1138,14 @@ int launch_acc_multi(const AccSegments& seg, const PayloadPtrs& pl, int k, bool 
     return launch_status();
 }
 
-uint32_t grid_for_items(uint64_t items)
+// Bands per workgroup of the band kernels, and the launch's workgroup count (0: out of range).
+uint32_t bands_grid(uint64_t n_rows, uint64_t n_cols, uint64_t range, uint32_t* bands_per_wg)
 {
-    uint64_t blocks = (items + kBlock2D - 1) / kBlock2D;
-    const uint64_t cap = (uint64_t)compute_units() * 64;
-    if (blocks > cap) blocks = cap;
-    return (uint32_t)(blocks ? blocks : 1);
+    const uint64_t m = n_rows / 16 + (n_rows % 16 ? 1 : 0);
+    const uint64_t per = range / (16 * n_cols);
+    *bands_per_wg = (uint32_t)(per ? per : 1);
+    const uint64_t blocks = (m + *bands_per_wg - 1) / *bands_per_wg;
+    return blocks > 0x7FFFFFFFull ? 0u : (uint32_t)blocks;
 }
 
 // n_rows * n_cols with overflow check
@@ -1095,21 +1235,38 @@ int nklq_quantize_f32(const float* g, const float* r_in, float* r_out, uint32_t*
         return dispatch_quant_flat(g, r_in, r_out, c, total, thrd, add, al, s);
     }
     const uint64_t m = n_rows / 16 + (n_rows % 16 ? 1 : 0);
-    if (n_cols < kNarrowColumns) {
-        const uint64_t items = m * n_cols;
-        const uint32_t grid = grid_for_items(items);
-        if (add)
-            hipLaunchKernelGGL((quant_2d_kernel<true>), dim3(grid), dim3(kBlock2D), 0, s, g, r_in,
-                               r_out, c, n_rows, n_cols, items, thrd);
-        else
-            hipLaunchKernelGGL((quant_2d_kernel<false>), dim3(grid), dim3(kBlock2D), 0, s, g, r_in,
-                               r_out, c, n_rows, n_cols, items, thrd);
+    if (n_cols <= kBandsMaxColumns) {
+        uint32_t per;
+        const uint32_t grid = bands_grid(n_rows, n_cols, kBandsRangeQuant, &per);
+        if (grid == 0) return NKLQ_ERANGE;
+        const uint32_t k32 = (uint32_t)n_cols;
+        const uint32_t inv = (uint32_t)(0x100000000ull / k32) + 1u;
+        // quads are laid out from a 16-byte boundary of r_out; g and r_in load as aligned vectors when
+        // they sit at the same offset from one
+        const uintptr_t ph = reinterpret_cast<uintptr_t>(r_out) & 15u;
+        const bool same = (reinterpret_cast<uintptr_t>(g) & 15u) == ph &&
+                          (!add || (reinterpret_cast<uintptr_t>(r_in) & 15u) == ph);
+#define NKLQ_QB(ADD, NT, AL)                                                                          \
+    hipLaunchKernelGGL((quant_bands_kernel<ADD, NT, AL>), dim3(grid), dim3(kBandsBlock), 0, s, g, r_in, r_out, \
+                       c, n_rows, k32, per, inv, thrd)
+        switch ((add ? 4 : 0) | (g_nontemporal ? 2 : 0) | (same ? 1 : 0)) {
+            case 7: NKLQ_QB(true, true, true); break;
+            case 6: NKLQ_QB(true, true, false); break;
+            case 5: NKLQ_QB(true, false, true); break;
+            case 4: NKLQ_QB(true, false, false); break;
+            case 3: NKLQ_QB(false, true, true); break;
+            case 2: NKLQ_QB(false, true, false); break;
+            case 1: NKLQ_QB(false, false, true); break;
+            default: NKLQ_QB(false, false, false); break;
+        }
+#undef NKLQ_QB
         return launch_status();
     }
     const bool al = (n_cols % 4 == 0) && aligned16(g) && aligned16(r_out) && (!add || aligned16(r_in));
     const uint64_t col_tiles = (n_cols + 255) / 256;
-    if (col_tiles > 0x7FFFFFFFull || m > 0x7FFFFFFFull / col_tiles) return NKLQ_ERANGE;
-    const dim3 grid((uint32_t)(m * col_tiles)), block(kRowsBlock);
+    const uint64_t m8 = (m + 7) / 8 * 8;  // word rows are dealt to the XCDs in groups of 8
+    if (col_tiles > 0x7FFFFFFFull || m8 > 0x7FFFFFFFull / col_tiles) return NKLQ_ERANGE;
+    const dim3 grid((uint32_t)(m8 * col_tiles)), block(kRowsBlock);
 #define NKLQ_Q2(ADD, NT, AL)                                                                         \
     hipLaunchKernelGGL((quant_2d_rows_kernel<ADD, NT, AL>), grid, block, 0, s, g, r_in, r_out, c, n_rows, \
                        n_cols, (uint32_t)col_tiles, thrd)
@@ -1141,23 +1298,33 @@ int nklq_dequantize_f32(float* out, const uint32_t* c, uint64_t n_rows, uint64_t
         return dispatch_deq_flat(out, c, total, thrd, s);
     }
     const uint64_t m = n_rows / 16 + (n_rows % 16 ? 1 : 0);
-    if (n_cols < kNarrowColumns) {
-        const uint64_t items = m * n_cols;
-        hipLaunchKernelGGL((deq_2d_kernel), dim3(grid_for_items(items)), dim3(kBlock2D), 0, s, out, c,
-                           n_rows, n_cols, items, thrd);
+    if (n_cols <= kBandsMaxColumns) {
+        uint32_t per;
+        const uint32_t grid = bands_grid(n_rows, n_cols, kBandsRangeDecode, &per);
+        if (grid == 0) return NKLQ_ERANGE;
+        const uint32_t k32 = (uint32_t)n_cols;
+        const uint32_t inv = (uint32_t)(0x100000000ull / k32) + 1u;
+        if (g_nontemporal)
+            hipLaunchKernelGGL((deq_bands_kernel<true>), dim3(grid), dim3(kBandsBlock), 0, s, out, c, n_rows,
+                               k32, per, inv, thrd);
+        else
+            hipLaunchKernelGGL((deq_bands_kernel<false>), dim3(grid), dim3(kBandsBlock), 0, s, out, c, n_rows,
+                               k32, per, inv, thrd);
         return launch_status();
     }
-    const bool al = (n_cols % 4 == 0) && aligned16(out) && aligned16(c);
-    const uint64_t col_tiles = (n_cols + 255) / 256;
-    if (col_tiles > 0x7FFFFFFFull || m > 0x7FFFFFFFull / col_tiles) return NKLQ_ERANGE;
-    const dim3 grid((uint32_t)(m * col_tiles)), block(kRowsBlock);
-#define NKLQ_D2(NT, AL)                                                                            \
-    hipLaunchKernelGGL((deq_2d_rows_kernel<NT, AL>), grid, block, 0, s, out, c, n_rows, n_cols, \
+    // rows that all start on a 128-byte line (and 16-byte aligned words) take the plain form
+    const bool plain = (n_cols % 32 == 0) && (reinterpret_cast<uintptr_t>(out) & 127u) == 0 && aligned16(c);
+    const uint64_t col_tiles = ((plain ? n_cols : n_cols + 31) + 255) / 256;
+    const uint64_t m8 = (m + 7) / 8 * 8;  // word rows are dealt to the XCDs in groups of 8
+    if (col_tiles > 0x7FFFFFFFull || m8 > 0x7FFFFFFFull / col_tiles) return NKLQ_ERANGE;
+    const dim3 grid((uint32_t)(m8 * col_tiles)), block(kRowsBlock);
+#define NKLQ_D2(NT, SHIFT)                                                                        \
+    hipLaunchKernelGGL((deq_2d_rows_kernel<NT, SHIFT>), grid, block, 0, s, out, c, n_rows, n_cols, \
                        (uint32_t)col_tiles, thrd)
-    if (g_nontemporal && al) NKLQ_D2(true, true);
-    else if (g_nontemporal) NKLQ_D2(true, false);
-    else if (al) NKLQ_D2(false, true);
-    else NKLQ_D2(false, false);
+    if (g_nontemporal && plain) NKLQ_D2(true, false);
+    else if (g_nontemporal) NKLQ_D2(true, true);
+    else if (plain) NKLQ_D2(false, false);
+    else NKLQ_D2(false, true);
 #undef NKLQ_D2
     return launch_status();
 }

@@ -127,6 +127,45 @@ def test_matrix_layout(n, k):
     assert_bits_equal(gpu_dequantize(junk, n, 0.5, k=k), oracle.c.dequantize(junk, n, 0.5))
 
 
+@pytest.mark.parametrize("n,k", [(5000, 3), (2003, 17), (700, 255), (100, 257), (130, 511), (40, 1023), (40, 1024),
+                                 (40, 1025), (33, 1030), (50, 4099), (20, 8191), (129, 2048), (16, 1000)])
+@pytest.mark.parametrize("og,orr,oc", [(0, 0, 0), (1, 1, 1), (3, 2, 0), (0, 1, 3)])
+def test_matrix_forms_inside_larger_buffers(n, k, og, orr, oc):
+    """Every column regime (bands of a few columns, one band per workgroup, row tiles; k a multiple
+    of 32, of 4, odd) with the matrices starting at any element of larger buffers; nothing outside
+    the views may be written."""
+    rng = np.random.default_rng(n * 31 + k + og + 2 * orr + 4 * oc)
+    thrd = 0.01
+    A = rng.normal(0, 0.01, (n, k)).astype(np.float32)
+    A.reshape(-1)[:: 37] = np.float32(thrd)  # exact hits
+    R0 = rng.normal(0, 0.004, (n, k)).astype(np.float32)
+    m = (n + 15) // 16
+    gbuf = torch.zeros(n * k + 8, device="cuda")
+    rbuf = torch.full((n * k + 8,), 7.0, device="cuda")
+    cbuf = torch.full((m * k + 8,), -1, dtype=torch.int32, device="cuda")
+    dA = gbuf[og:og + n * k].view(n, k)
+    dR = rbuf[orr:orr + n * k].view(n, k)
+    dC = cbuf[oc:oc + m * k].view(m, k)
+    dA.copy_(torch.from_numpy(A))
+    for fused in (False, True):
+        if fused:
+            dR.copy_(torch.from_numpy(R0))
+        q.cu_fn_matrix_quantize_e(dA, dC, dR, thrd, add_residual=fused)
+        want_c, want_r = oracle.c.quantize(A, thrd, R_in=R0 if fused else None)
+        what = f"n={n} k={k} offsets={og},{orr},{oc} fused={fused}"
+        assert_words_equal(host_words(dC), want_c, what)
+        assert_bits_equal(dR.cpu().numpy(), want_r, what)
+        assert float(rbuf[:orr].sum()) == 7.0 * orr and float(rbuf[orr + n * k:].sum()) == 7.0 * (8 - orr), what
+        assert int(cbuf[:oc].sum()) == -oc and int(cbuf[oc + m * k:].sum()) == -(8 - oc), what
+        assert np.array_equal(dA.cpu().numpy().view(np.uint32), A.view(np.uint32)), what
+    junk = rng.integers(0, 2 ** 32, size=(m, k), dtype=np.uint64).astype(np.uint32)
+    dC.copy_(dev(junk))
+    rbuf.fill_(9.0)
+    q.cu_fn_matrix_dequantize_e(dR, dC, None, thrd)
+    assert_bits_equal(dR.cpu().numpy(), oracle.c.dequantize(junk, n, thrd), f"decode n={n} k={k}")
+    assert float(rbuf[:orr].sum()) == 9.0 * orr and float(rbuf[orr + n * k:].sum()) == 9.0 * (8 - orr)
+
+
 def test_in_place_forms():
     """R may be A itself (plain), and the fused step updates R in place."""
     rng = np.random.default_rng(99)
