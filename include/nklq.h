@@ -6,8 +6,12 @@
  * types.  Every pointer marked "device" must be memory the current HIP device
  * can address; `stream` is a hipStream_t passed as an opaque pointer (NULL =
  * the device's default stream).  All entry points are asynchronous on
- * `stream`, allocate nothing, keep no state between calls (other than the
- * nklq_tune knobs) and may be called from several host threads at once.
+ * `stream`, allocate no device memory and keep no state between calls other
+ * than the nklq_tune knobs.  They may be called from several host threads at
+ * once, also while another thread changes a knob: the knobs are atomics and a
+ * call works from the one snapshot it takes on entry.  The int return value
+ * of a launch is that launch's own status, not the runtime's sticky
+ * "last error".
  *
  * Bit layout (necklace/cuda/quantize.py:8-13, :34-51): codes are 2 bits,
  * 01 = value >= t, 10 = value <= -t, 00 = in between, 16 codes per 32-bit
@@ -35,7 +39,10 @@ extern "C" {
 #define NKLQ_ENULL (-1)   /* a required pointer is NULL */
 #define NKLQ_EALIGN (-2)  /* a pointer is not 4-byte aligned */
 #define NKLQ_ERANGE (-3)  /* a size or count is out of range */
-#define NKLQ_EALIAS (-4)  /* outputs overlap in a way the call cannot honour */
+#define NKLQ_EALIAS (-4)  /* the byte range of an output overlaps another buffer of the call; only an
+                             output that coincides exactly with an input (r_out == r_in, r_out == g)
+                             is allowed.  Checked over the full extents, across all vectors of the
+                             *_multi_* calls, before anything is launched */
 
 /*
  * Threshold-quantize an fp32 matrix to 2-bit codes and write the residual.
@@ -47,7 +54,7 @@ extern "C" {
  *          read only when add_residual != 0 (may be NULL otherwise)
  *   r_out  device, fp32 same shape: the matrix R of the reference (every
  *          element is written).  May be the same pointer as r_in (in-place
- *          error feedback) or as g; any other overlap is undefined.
+ *          error feedback) or as g; any other overlap returns NKLQ_EALIAS.
  *   c      device, uint32 [ceil(n_rows/16), n_cols] row-major: the matrix C
  *          (every word is overwritten, whatever it held)
  *   thrd   the threshold; it crosses as C float, i.e. rounded to fp32 exactly
@@ -140,9 +147,10 @@ int nklq_version(void);
 /*
  * Launch-geometry knobs, the counterpart of the reference wrapper's bpg/tpb
  * keyword arguments (necklace/cuda/quantize.py:98,120).  Results never depend
- * on them; they apply to the flat kernels of every later call in the process.
- * Returns the previous value, or NKLQ_ERANGE for an unknown knob or a value
- * outside its set.  value < 0 only queries.
+ * on them; they apply to the flat kernels of every later call in the process
+ * (the sum over payloads only has its interleave knob).  Returns the previous
+ * value, or NKLQ_ERANGE for an unknown knob or a value outside its set.
+ * value < 0 only queries.  Safe to call while other threads launch.
  */
 #define NKLQ_TUNE_CHUNKS_PER_WAVE 0      /* 256-element chunks per wave: 1, 2 or 4 */
 #define NKLQ_TUNE_WORKGROUP_SIZE 1       /* threads per workgroup: 64, 128, 256, 512 or 1024 */

@@ -31,6 +31,12 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <algorithm>
+#include <atomic>
+#include <tuple>
+#include <utility>
+#include <vector>
+
 #include "nklq.h"
 
 namespace {
@@ -880,27 +886,95 @@ __global__ __launch_bounds__(BLOCK) void copy_kernel(float* dst, const float* sr
 
 // ---------------------------------------------------------------- host side
 
-// Launch-geometry knobs (results never depend on them); defaults from a sweep on MI355X.
-int g_chunks_per_wave = 1;  // 1, 2 or 4
-int g_block = 256;          // 64, 128, 256, 512 or 1024 threads
-int g_nontemporal = 1;
-int g_xcd_shift = 2;        // quantize/copy: chunks interleaved over 2^g_xcd_shift workgroups
-int g_xcd_shift_decode = 0; // the same for dequantize (write-dominated: contiguous wins)
-int g_xcd_shift_acc = 3;    // the same for the sum over payloads (tiles of 1024 elements, dealt over all 8 XCDs)
+// Launch-geometry knobs (results never depend on them); defaults from a sweep on MI355X.  They
+// are process-wide and may be changed by one host thread while others launch: every entry point
+// takes one snapshot of them when it is called and uses only that.
+struct Knobs {
+    int chunks_per_wave;  // 1, 2 or 4
+    int block;            // 64, 128, 256, 512 or 1024 threads
+    int nontemporal;
+    int xcd_shift;        // quantize/copy: chunks interleaved over 2^xcd_shift workgroups
+    int xcd_shift_decode; // the same for dequantize (write-dominated: contiguous wins)
+    int xcd_shift_acc;    // the same for the sum over payloads (tiles of 1024 elements over all 8 XCDs)
+};
+constexpr int kKnobCount = 6;
+std::atomic<int> g_knobs[kKnobCount] = {{1}, {256}, {1}, {2}, {0}, {3}};
 
-int compute_units()
+thread_local Knobs tk;  // the calling thread's snapshot, taken on entry to an entry point
+
+inline void snapshot_knobs()
 {
-    static int cached[64] = {0};
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-    if (cached[dev] == 0) {
-        int cu = 0;
-        if (hipDeviceGetAttribute(&cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
-            cu <= 0)
-            cu = 256;
-        cached[dev] = cu;
+    tk.chunks_per_wave = g_knobs[NKLQ_TUNE_CHUNKS_PER_WAVE].load(std::memory_order_relaxed);
+    tk.block = g_knobs[NKLQ_TUNE_WORKGROUP_SIZE].load(std::memory_order_relaxed);
+    tk.nontemporal = g_knobs[NKLQ_TUNE_NONTEMPORAL].load(std::memory_order_relaxed);
+    tk.xcd_shift = g_knobs[NKLQ_TUNE_XCD_INTERLEAVE_LOG2].load(std::memory_order_relaxed);
+    tk.xcd_shift_decode = g_knobs[NKLQ_TUNE_XCD_INTERLEAVE_LOG2_DECODE].load(std::memory_order_relaxed);
+    tk.xcd_shift_acc = g_knobs[NKLQ_TUNE_XCD_INTERLEAVE_LOG2_ACCUMULATE].load(std::memory_order_relaxed);
+}
+
+// ---- kernel launch with the launch's own status
+//
+// hipLaunchKernel returns what THIS launch did; the runtime's "last error" is left alone unless the
+// launch failed (then it is cleared, since the failure is reported through the return value).
+thread_local int t_launch_status = NKLQ_OK;
+
+template <typename Tuple, size_t... I>
+inline void arg_pointers(Tuple& vals, void** out, std::index_sequence<I...>)
+{
+    ((out[I] = static_cast<void*>(&std::get<I>(vals))), ...);
+}
+
+template <typename... KArgs, typename... Args>
+inline void launch_kernel(void (*kernel)(KArgs...), dim3 grid, dim3 block, uint32_t lds_bytes, hipStream_t s,
+                          Args... args)
+{
+    static_assert(sizeof...(KArgs) == sizeof...(Args), "kernel argument count");
+    std::tuple<KArgs...> vals(static_cast<KArgs>(args)...);
+    void* ptrs[sizeof...(KArgs)];
+    arg_pointers(vals, ptrs, std::index_sequence_for<KArgs...>{});
+    const hipError_t e = hipLaunchKernel(reinterpret_cast<const void*>(kernel), grid, block, ptrs, lds_bytes, s);
+    if (e != hipSuccess) (void)hipGetLastError();
+    t_launch_status = e == hipSuccess ? NKLQ_OK : (int)e;
+}
+
+inline int launch_status() { return t_launch_status; }
+
+// ---- overlap checks
+//
+// Byte ranges of the buffers of a call.  An output may coincide EXACTLY with an input (the in-place
+// forms: r_out == r_in, r_out == g); any other overlap that involves an output is refused.
+struct Span {
+    uintptr_t lo, hi;
+    bool out;
+};
+
+inline Span span_of(const void* p, uint64_t bytes, bool out)
+{
+    const uintptr_t lo = reinterpret_cast<uintptr_t>(p);
+    return Span{lo, lo + (uintptr_t)bytes, out};
+}
+
+bool spans_conflict(std::vector<Span>& v)
+{
+    std::sort(v.begin(), v.end(), [](const Span& a, const Span& b) {
+        if (a.lo != b.lo) return a.lo < b.lo;
+        if (a.hi != b.hi) return a.hi < b.hi;
+        return a.out > b.out;  // of identical ranges the output comes first
+    });
+    uintptr_t end_out = 0, end_any = 0;  // furthest end among the outputs / all ranges seen so far
+    uintptr_t out_lo = 0, out_hi = 0;    // the latest output
+    for (size_t i = 0; i < v.size(); ++i) {
+        if (v[i].lo == v[i].hi) continue;
+        // inputs identical to the output sorted just before them are that output's in-place partners
+        const bool partner = !v[i].out && out_hi != 0 && v[i].lo == out_lo && v[i].hi == out_hi;
+        if (v[i].out) { out_lo = v[i].lo; out_hi = v[i].hi; }
+        if (!partner) {
+            if (v[i].out ? v[i].lo < end_any : v[i].lo < end_out) return true;
+        }
+        if (v[i].out && v[i].hi > end_out) end_out = v[i].hi;
+        if (v[i].hi > end_any) end_any = v[i].hi;
     }
-    return cached[dev];
+    return false;
 }
 
 struct FlatGrid {
@@ -926,23 +1000,17 @@ FlatGrid flat_grid(uint64_t n, int U, int block, int xcd_shift)
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 inline bool aligned4(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 3u) == 0; }
 
-inline int launch_status()
-{
-    const hipError_t e = hipGetLastError();
-    return e == hipSuccess ? NKLQ_OK : (int)e;
-}
-
 // ---- flat quantize dispatch: (U, BLOCK) -> (ALIGNED, ADD, NT)
 
 template <int U, int BLOCK>
 int launch_quant_flat(const float* g, const float* rin, float* rout, uint32_t* c, uint64_t n, float t,
                       bool add, bool al, hipStream_t s)
 {
-    const FlatGrid fg = flat_grid(n, U, BLOCK, g_xcd_shift);
+    const FlatGrid fg = flat_grid(n, U, BLOCK, tk.xcd_shift);
     if (fg.blocks == 0) return NKLQ_ERANGE;
-    const bool nt = g_nontemporal != 0;
+    const bool nt = tk.nontemporal != 0;
 #define NKLQ_Q(AL, ADD, NT)                                                                       \
-    hipLaunchKernelGGL((quant_flat_kernel<U, BLOCK, AL, ADD, NT>), dim3(fg.blocks), dim3(BLOCK), 0, \
+    launch_kernel((quant_flat_kernel<U, BLOCK, AL, ADD, NT>), dim3(fg.blocks), dim3(BLOCK), 0, \
                        s, g, rin, rout, c, n, fg.n_chunks, fg.has_tail, fg.xs, t)
     const int sel = (al ? 4 : 0) | (add ? 2 : 0) | (nt ? 1 : 0);
     switch (sel) {
@@ -962,12 +1030,12 @@ int launch_quant_flat(const float* g, const float* rin, float* rout, uint32_t* c
 template <int U, int BLOCK>
 int launch_deq_flat(float* out, const uint32_t* c, uint64_t n, float t, hipStream_t s)
 {
-    const FlatGrid fg = flat_grid(n, U, BLOCK, g_xcd_shift_decode);
+    const FlatGrid fg = flat_grid(n, U, BLOCK, tk.xcd_shift_decode);
     if (fg.blocks == 0) return NKLQ_ERANGE;
     const bool al = aligned16(out);
-    const bool nt = g_nontemporal != 0;
+    const bool nt = tk.nontemporal != 0;
 #define NKLQ_DEQ(AL, NT)                                                                        \
-    hipLaunchKernelGGL((deq_flat_kernel<U, BLOCK, AL, NT>), dim3(fg.blocks), dim3(BLOCK), 0, s, out, \
+    launch_kernel((deq_flat_kernel<U, BLOCK, AL, NT>), dim3(fg.blocks), dim3(BLOCK), 0, s, out, \
                        c, n, fg.n_chunks, fg.has_tail, fg.xs, t)
     if (al && nt) NKLQ_DEQ(true, true);
     else if (al) NKLQ_DEQ(true, false);
@@ -1013,7 +1081,7 @@ int launch_acc_flat(float* acc, const PayloadPtrs& pl, int k, uint64_t n, float 
 {
     const uint64_t n_tiles = n / kTile;
     const uint32_t has_tail = (n_tiles * kTile < n) ? 1u : 0u;
-    const uint32_t xs = (uint32_t)g_xcd_shift_acc;
+    const uint32_t xs = (uint32_t)tk.xcd_shift_acc;
     const uint64_t per_group = (uint64_t)(kAccBlock / kWave) << xs;
     const uint64_t work = ((n_tiles + per_group - 1) / per_group) << xs;
     if (work + has_tail > 0x7FFFFFFFull) return NKLQ_ERANGE;
@@ -1023,7 +1091,7 @@ int launch_acc_flat(float* acc, const PayloadPtrs& pl, int k, uint64_t n, float 
     const float th = -0.5f * t;
     const uint32_t pad = n_tiles >= kAccThrottleTiles ? kAccThrottleLdsBytes : 0u;
 #define NKLQ_ACC(K, AL, MIX)                                                                        \
-    hipLaunchKernelGGL((acc_flat_kernel<K, AL, MIX>), dim3(blocks), dim3(kAccBlock), pad, s, acc, pl, k, n, \
+    launch_kernel((acc_flat_kernel<K, AL, MIX>), dim3(blocks), dim3(kAccBlock), pad, s, acc, pl, k, n, \
                        n_tiles, has_tail, xs, t, th, accumulate)
     NKLQ_ACC_DISPATCH(NKLQ_ACC, k, al, mix);
 #undef NKLQ_ACC
@@ -1032,7 +1100,7 @@ int launch_acc_flat(float* acc, const PayloadPtrs& pl, int k, uint64_t n, float 
 
 // Expands to the call of FN<U, BLOCK, ...> for the current knob values.
 #define NKLQ_FOR_GEOMETRY(CALL)                                  \
-    switch (g_chunks_per_wave * 10000 + g_block) {               \
+    switch (tk.chunks_per_wave * 10000 + tk.block) {               \
         case 10064: return CALL(1, 64);                          \
         case 10128: return CALL(1, 128);                         \
         case 10256: return CALL(1, 256);                         \
@@ -1069,13 +1137,13 @@ int dispatch_deq_flat(float* out, const uint32_t* c, uint64_t n, float t, hipStr
 template <int U, int BLOCK>
 int launch_copy(float* dst, const float* src, uint64_t n, hipStream_t s)
 {
-    const FlatGrid fg = flat_grid(n, U, BLOCK, g_xcd_shift);
+    const FlatGrid fg = flat_grid(n, U, BLOCK, tk.xcd_shift);
     if (fg.blocks == 0) return NKLQ_ERANGE;
-    if (g_nontemporal)
-        hipLaunchKernelGGL((copy_kernel<U, BLOCK, true>), dim3(fg.blocks), dim3(BLOCK), 0, s, dst, src,
+    if (tk.nontemporal)
+        launch_kernel((copy_kernel<U, BLOCK, true>), dim3(fg.blocks), dim3(BLOCK), 0, s, dst, src,
                            n, fg.n_chunks, fg.has_tail, fg.xs);
     else
-        hipLaunchKernelGGL((copy_kernel<U, BLOCK, false>), dim3(fg.blocks), dim3(BLOCK), 0, s, dst,
+        launch_kernel((copy_kernel<U, BLOCK, false>), dim3(fg.blocks), dim3(BLOCK), 0, s, dst,
                            src, n, fg.n_chunks, fg.has_tail, fg.xs);
     return launch_status();
 }
@@ -1100,12 +1168,12 @@ bool multi_grid(uint64_t total, uint32_t xs, uint32_t* blocks)
 int launch_quant_multi(const QuantSegments& seg, bool al, bool add, float t, hipStream_t s)
 {
     uint32_t blocks;
-    const uint32_t xs = (uint32_t)g_xcd_shift;
+    const uint32_t xs = (uint32_t)tk.xcd_shift;
     if (!multi_grid(seg.first[seg.count], xs, &blocks)) return NKLQ_ERANGE;
     if (blocks == 0) return NKLQ_OK;
-    const bool nt = g_nontemporal != 0;
+    const bool nt = tk.nontemporal != 0;
 #define NKLQ_QM(AL, ADD, NT) \
-    hipLaunchKernelGGL((quant_multi_kernel<AL, ADD, NT>), dim3(blocks), dim3(256), 0, s, seg, xs, t)
+    launch_kernel((quant_multi_kernel<AL, ADD, NT>), dim3(blocks), dim3(256), 0, s, seg, xs, t)
     switch ((al ? 4 : 0) | (add ? 2 : 0) | (nt ? 1 : 0)) {
         case 7: NKLQ_QM(true, true, true); break;
         case 6: NKLQ_QM(true, true, false); break;
@@ -1124,14 +1192,14 @@ int launch_acc_multi(const AccSegments& seg, const PayloadPtrs& pl, int k, bool 
                      int accumulate, float divisor, hipStream_t s)
 {
     uint32_t blocks;
-    const uint32_t xs = (uint32_t)g_xcd_shift_acc;
+    const uint32_t xs = (uint32_t)tk.xcd_shift_acc;
     if (!multi_grid(seg.first[seg.count], xs, &blocks)) return NKLQ_ERANGE;
     if (blocks == 0) return NKLQ_OK;
     const bool mix = mix_ok(t);
     const float th = -0.5f * t;
     const uint32_t pad = seg.first[seg.count] >= kAccThrottleTiles ? kAccThrottleLdsBytes : 0u;
 #define NKLQ_AM(K, AL, MIX)                                                                           \
-    hipLaunchKernelGGL((acc_multi_kernel<K, AL, MIX>), dim3(blocks), dim3(kAccBlock), pad, s, seg, pl, k, xs, \
+    launch_kernel((acc_multi_kernel<K, AL, MIX>), dim3(blocks), dim3(kAccBlock), pad, s, seg, pl, k, xs, \
                        t, th, accumulate, divisor)
     NKLQ_ACC_DISPATCH(NKLQ_AM, k, al, mix);
 #undef NKLQ_AM
@@ -1185,18 +1253,8 @@ const char* nklq_strerror(int code)
 
 int nklq_tune(int which, int value)
 {
-    int* slot = nullptr;
-    switch (which) {
-        case NKLQ_TUNE_CHUNKS_PER_WAVE: slot = &g_chunks_per_wave; break;
-        case NKLQ_TUNE_WORKGROUP_SIZE: slot = &g_block; break;
-        case NKLQ_TUNE_NONTEMPORAL: slot = &g_nontemporal; break;
-        case NKLQ_TUNE_XCD_INTERLEAVE_LOG2: slot = &g_xcd_shift; break;
-        case NKLQ_TUNE_XCD_INTERLEAVE_LOG2_DECODE: slot = &g_xcd_shift_decode; break;
-        case NKLQ_TUNE_XCD_INTERLEAVE_LOG2_ACCUMULATE: slot = &g_xcd_shift_acc; break;
-        default: return NKLQ_ERANGE;
-    }
-    const int prev = *slot;
-    if (value < 0) return prev;
+    if (which < 0 || which >= kKnobCount) return NKLQ_ERANGE;
+    if (value < 0) return g_knobs[which].load(std::memory_order_relaxed);
     switch (which) {
         case NKLQ_TUNE_CHUNKS_PER_WAVE:
             if (value != 1 && value != 2 && value != 4) return NKLQ_ERANGE;
@@ -1212,8 +1270,7 @@ int nklq_tune(int which, int value)
             if (value > 6) return NKLQ_ERANGE;
             break;
     }
-    *slot = value;
-    return prev;
+    return g_knobs[which].exchange(value, std::memory_order_relaxed);
 }
 
 int nklq_quantize_f32(const float* g, const float* r_in, float* r_out, uint32_t* c,
@@ -1225,9 +1282,16 @@ int nklq_quantize_f32(const float* g, const float* r_in, float* r_out, uint32_t*
     if (!g || !r_out || !c || (add_residual && !r_in)) return NKLQ_ENULL;
     if (!aligned4(g) || !aligned4(r_out) || !aligned4(c) || (add_residual && !aligned4(r_in)))
         return NKLQ_EALIGN;
-    if ((const void*)c == (const void*)g || (const void*)c == (const void*)r_out) return NKLQ_EALIAS;
-    hipStream_t s = (hipStream_t)stream;
     const bool add = add_residual != 0;
+    {
+        std::vector<Span> spans = {span_of(r_out, 4 * total, true),
+                                   span_of(c, 4 * nklq_packed_words(n_rows, n_cols), true),
+                                   span_of(g, 4 * total, false)};
+        if (add) spans.push_back(span_of(r_in, 4 * total, false));
+        if (spans_conflict(spans)) return NKLQ_EALIAS;
+    }
+    snapshot_knobs();
+    hipStream_t s = (hipStream_t)stream;
     if (!add) r_in = g;  // never read; keeps the argument a valid address
 
     if (n_cols == 1) {
@@ -1247,9 +1311,9 @@ int nklq_quantize_f32(const float* g, const float* r_in, float* r_out, uint32_t*
         const bool same = (reinterpret_cast<uintptr_t>(g) & 15u) == ph &&
                           (!add || (reinterpret_cast<uintptr_t>(r_in) & 15u) == ph);
 #define NKLQ_QB(ADD, NT, AL)                                                                          \
-    hipLaunchKernelGGL((quant_bands_kernel<ADD, NT, AL>), dim3(grid), dim3(kBandsBlock), 0, s, g, r_in, r_out, \
+    launch_kernel((quant_bands_kernel<ADD, NT, AL>), dim3(grid), dim3(kBandsBlock), 0, s, g, r_in, r_out, \
                        c, n_rows, k32, per, inv, thrd)
-        switch ((add ? 4 : 0) | (g_nontemporal ? 2 : 0) | (same ? 1 : 0)) {
+        switch ((add ? 4 : 0) | (tk.nontemporal ? 2 : 0) | (same ? 1 : 0)) {
             case 7: NKLQ_QB(true, true, true); break;
             case 6: NKLQ_QB(true, true, false); break;
             case 5: NKLQ_QB(true, false, true); break;
@@ -1268,9 +1332,9 @@ int nklq_quantize_f32(const float* g, const float* r_in, float* r_out, uint32_t*
     if (col_tiles > 0x7FFFFFFFull || m8 > 0x7FFFFFFFull / col_tiles) return NKLQ_ERANGE;
     const dim3 grid((uint32_t)(m8 * col_tiles)), block(kRowsBlock);
 #define NKLQ_Q2(ADD, NT, AL)                                                                         \
-    hipLaunchKernelGGL((quant_2d_rows_kernel<ADD, NT, AL>), grid, block, 0, s, g, r_in, r_out, c, n_rows, \
+    launch_kernel((quant_2d_rows_kernel<ADD, NT, AL>), grid, block, 0, s, g, r_in, r_out, c, n_rows, \
                        n_cols, (uint32_t)col_tiles, thrd)
-    switch ((add ? 4 : 0) | (g_nontemporal ? 2 : 0) | (al ? 1 : 0)) {
+    switch ((add ? 4 : 0) | (tk.nontemporal ? 2 : 0) | (al ? 1 : 0)) {
         case 7: NKLQ_Q2(true, true, true); break;
         case 6: NKLQ_Q2(true, true, false); break;
         case 5: NKLQ_Q2(true, false, true); break;
@@ -1292,7 +1356,12 @@ int nklq_dequantize_f32(float* out, const uint32_t* c, uint64_t n_rows, uint64_t
     if (total == 0) return NKLQ_OK;
     if (!out || !c) return NKLQ_ENULL;
     if (!aligned4(out) || !aligned4(c)) return NKLQ_EALIGN;
-    if ((const void*)c == (const void*)out) return NKLQ_EALIAS;
+    {
+        std::vector<Span> spans = {span_of(out, 4 * total, true),
+                                   span_of(c, 4 * nklq_packed_words(n_rows, n_cols), false)};
+        if (spans_conflict(spans)) return NKLQ_EALIAS;
+    }
+    snapshot_knobs();
     hipStream_t s = (hipStream_t)stream;
     if (n_cols == 1) {
         return dispatch_deq_flat(out, c, total, thrd, s);
@@ -1304,11 +1373,11 @@ int nklq_dequantize_f32(float* out, const uint32_t* c, uint64_t n_rows, uint64_t
         if (grid == 0) return NKLQ_ERANGE;
         const uint32_t k32 = (uint32_t)n_cols;
         const uint32_t inv = (uint32_t)(0x100000000ull / k32) + 1u;
-        if (g_nontemporal)
-            hipLaunchKernelGGL((deq_bands_kernel<true>), dim3(grid), dim3(kBandsBlock), 0, s, out, c, n_rows,
+        if (tk.nontemporal)
+            launch_kernel((deq_bands_kernel<true>), dim3(grid), dim3(kBandsBlock), 0, s, out, c, n_rows,
                                k32, per, inv, thrd);
         else
-            hipLaunchKernelGGL((deq_bands_kernel<false>), dim3(grid), dim3(kBandsBlock), 0, s, out, c, n_rows,
+            launch_kernel((deq_bands_kernel<false>), dim3(grid), dim3(kBandsBlock), 0, s, out, c, n_rows,
                                k32, per, inv, thrd);
         return launch_status();
     }
@@ -1319,10 +1388,10 @@ int nklq_dequantize_f32(float* out, const uint32_t* c, uint64_t n_rows, uint64_t
     if (col_tiles > 0x7FFFFFFFull || m8 > 0x7FFFFFFFull / col_tiles) return NKLQ_ERANGE;
     const dim3 grid((uint32_t)(m8 * col_tiles)), block(kRowsBlock);
 #define NKLQ_D2(NT, SHIFT)                                                                        \
-    hipLaunchKernelGGL((deq_2d_rows_kernel<NT, SHIFT>), grid, block, 0, s, out, c, n_rows, n_cols, \
+    launch_kernel((deq_2d_rows_kernel<NT, SHIFT>), grid, block, 0, s, out, c, n_rows, n_cols, \
                        (uint32_t)col_tiles, thrd)
-    if (g_nontemporal && plain) NKLQ_D2(true, false);
-    else if (g_nontemporal) NKLQ_D2(true, true);
+    if (tk.nontemporal && plain) NKLQ_D2(true, false);
+    else if (tk.nontemporal) NKLQ_D2(true, true);
     else if (plain) NKLQ_D2(false, false);
     else NKLQ_D2(false, true);
 #undef NKLQ_D2
@@ -1336,11 +1405,16 @@ int nklq_dequant_accumulate_f32(float* acc, const uint32_t* const* payloads, int
     if (n == 0) return NKLQ_OK;
     if (!acc || !payloads) return NKLQ_ENULL;
     if (!aligned4(acc)) return NKLQ_EALIGN;
-    for (int p = 0; p < k_payloads; ++p) {
-        if (!payloads[p]) return NKLQ_ENULL;
-        if (!aligned4(payloads[p])) return NKLQ_EALIGN;
-        if ((const void*)payloads[p] == (const void*)acc) return NKLQ_EALIAS;
+    {
+        std::vector<Span> spans = {span_of(acc, 4 * n, true)};
+        for (int p = 0; p < k_payloads; ++p) {
+            if (!payloads[p]) return NKLQ_ENULL;
+            if (!aligned4(payloads[p])) return NKLQ_EALIGN;
+            spans.push_back(span_of(payloads[p], 4 * nklq_packed_words(n, 1), false));
+        }
+        if (spans_conflict(spans)) return NKLQ_EALIAS;
     }
+    snapshot_knobs();
     hipStream_t s = (hipStream_t)stream;
     if (k_payloads == 1 && !accumulate && (__builtin_bit_cast(uint32_t, thrd) & 0x7FFFFFFFu) != 0) {
         // +0.0 + d is d for d in {+t, -t, +0.0} unless t is a zero (then -t = -0.0 would become
@@ -1371,10 +1445,20 @@ int nklq_quantize_multi_f32(int count, const float* const* g, float* const* r, u
         if (n[i] == 0) continue;
         if (!g[i] || !r[i] || !c[i]) return NKLQ_ENULL;
         if (!aligned4(g[i]) || !aligned4(r[i]) || !aligned4(c[i])) return NKLQ_EALIGN;
-        if ((const void*)c[i] == (const void*)g[i] || (const void*)c[i] == (const void*)r[i])
-            return NKLQ_EALIAS;
         if (n[i] / kChunk + 1 > 0x7FFFFFFFull) return NKLQ_ERANGE;
     }
+    {
+        std::vector<Span> spans;
+        spans.reserve(3 * (size_t)count);
+        for (int i = 0; i < count; ++i) {
+            if (n[i] == 0) continue;
+            spans.push_back(span_of(r[i], 4 * n[i], true));
+            spans.push_back(span_of(c[i], 4 * nklq_packed_words(n[i], 1), true));
+            spans.push_back(span_of(g[i], 4 * n[i], false));
+        }
+        if (spans_conflict(spans)) return NKLQ_EALIAS;
+    }
+    snapshot_knobs();
     hipStream_t s = (hipStream_t)stream;
     int i = 0;
     while (i < count) {
@@ -1425,6 +1509,24 @@ int nklq_dequant_accumulate_multi_f32(int count, float* const* acc, const uint64
         if (!aligned4(acc[i])) return NKLQ_EALIGN;
         if (n[i] / kTile + 1 > 0x7FFFFFFFull) return NKLQ_ERANGE;
     }
+    {
+        // every payload is read between its lowest and highest word any vector uses
+        uint64_t w_lo = UINT64_MAX, w_hi = 0;
+        std::vector<Span> spans;
+        spans.reserve((size_t)count + (size_t)k_payloads);
+        for (int i = 0; i < count; ++i) {
+            if (n[i] == 0) continue;
+            spans.push_back(span_of(acc[i], 4 * n[i], true));
+            if (word_offset[i] < w_lo) w_lo = word_offset[i];
+            const uint64_t end = word_offset[i] + nklq_packed_words(n[i], 1);
+            if (end > w_hi) w_hi = end;
+        }
+        if (w_lo < w_hi)
+            for (int p = 0; p < k_payloads; ++p)
+                spans.push_back(span_of(payload_base[p] + w_lo, 4 * (w_hi - w_lo), false));
+        if (spans_conflict(spans)) return NKLQ_EALIAS;
+    }
+    snapshot_knobs();
     hipStream_t s = (hipStream_t)stream;
     int acc_flag = accumulate ? 1 : 0;
     for (int first_p = 0; first_p < k_payloads; first_p += NKLQ_MAX_PAYLOADS_PER_LAUNCH) {
@@ -1472,6 +1574,11 @@ int nklq_copy_f32(float* dst, const float* src, uint64_t n, void* stream)
     if (n == 0) return NKLQ_OK;
     if (!dst || !src) return NKLQ_ENULL;
     if (!aligned16(dst) || !aligned16(src)) return NKLQ_EALIGN;
+    {
+        std::vector<Span> spans = {span_of(dst, 4 * n, true), span_of(src, 4 * n, false)};
+        if (spans_conflict(spans)) return NKLQ_EALIAS;
+    }
+    snapshot_knobs();
     return dispatch_copy(dst, src, n, (hipStream_t)stream);
 }
 

@@ -67,9 +67,41 @@ def test_argument_errors_are_reported_without_a_launch():
         _lib.check(-2)
 
 
+def test_partial_overlaps_are_refused_without_a_launch():
+    """Byte-range checks: an output may coincide exactly with an input (the in-place forms), any
+    other overlap that involves an output is NKLQ_EALIAS.  Every case returns before a launch."""
+    L = _lib.lib()
+    vp, u64 = ct.c_void_p, ct.c_uint64
+    base = 0x100000
+    n = 4096                      # 16 KiB of fp32, 256 words (1 KiB) of codes
+    g, r, c = base, base + 0x10000, base + 0x20000
+    q = lambda g_, rin, rout, c_, add=1: L.nklq_quantize_f32(g_, rin, rout, c_, n, 1, 0.5, add, None)
+    assert q(g, r, r, g + 4 * 100) == -4            # codes land in the middle of g
+    assert q(g, r, r, r + 4 * n - 8) == -4          # codes straddle the end of the residual
+    assert q(g, r, g + 8, c) == -4                  # residual out shifted against g
+    assert q(g, r, r + 4, c) == -4                  # residual out shifted against residual in
+    assert q(g, r, r, r - 1020) == -4               # the last word of c is the first float of the residual
+    assert L.nklq_dequantize_f32(g, g + 4 * (n - 1), n, 1, 0.5, None) == -4     # words start inside out
+    arr = (vp * 2)(c, g + 64)
+    assert L.nklq_dequant_accumulate_f32(g, arr, 2, n, 0.5, 0, None) == -4      # second payload inside acc
+    # many vectors: an output of one vector on top of a buffer of another
+    gs, rs, cs = (vp * 2)(g, g + 0x4000), (vp * 2)(r, r + 0x4000), (vp * 2)(c, r + 0x4000 - 16)
+    ns = (u64 * 2)(n, n)
+    assert L.nklq_quantize_multi_f32(2, gs, rs, cs, ns, 0.5, 1, None) == -4     # c[1] ends inside r[1]
+    cs2 = (vp * 2)(c, c + 512)
+    assert L.nklq_quantize_multi_f32(2, gs, rs, cs2, ns, 0.5, 1, None) == -4    # c[1] starts inside c[0]
+    accs = (vp * 2)(g, g + 4 * n - 4)
+    woff = (u64 * 2)(0, 256)
+    bases = (vp * 1)(c)
+    assert L.nklq_dequant_accumulate_multi_f32(2, accs, ns, woff, bases, 1, 0.5, 0, 1.0, None) == -4  # acc[1] over acc[0]
+    accs = (vp * 2)(g, g + 0x4000)
+    bases = (vp * 1)(g + 0x4000 + 4 * n - 1024)
+    assert L.nklq_dequant_accumulate_multi_f32(2, accs, ns, woff, bases, 1, 0.5, 0, 1.0, None) == -4  # message over acc[1]
+
+
 def test_tune_knobs_round_trip():
     for which, good, bad in ((0, (1, 2, 4), 3), (1, (64, 128, 256, 512, 1024), 96), (2, (0, 1), None),
-                             (3, (0, 1, 2, 3, 4, 5, 6), 7), (4, (0, 3, 6), 7)):
+                             (3, (0, 1, 2, 3, 4, 5, 6), 7), (4, (0, 3, 6), 7), (5, (0, 3, 6), 7)):
         before = _lib.tune(which)
         for v in good:
             _lib.tune(which, v)

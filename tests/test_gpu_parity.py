@@ -44,12 +44,22 @@ def test_kat_vectors_on_gpu(kat):
         t = float(bits_to_f32([v["thrd_bits"]])[0])
         words = np.array([int(h, 16) for h in v["words"]], dtype=np.uint32)
         assert_bits_equal(gpu_dequantize(words, v["n"], t), bits_to_f32(v["out_bits"]), v["name"])
+    nan_bits = lambda hs: bits_to_f32([("7FC00000" if h == "NAN" else h) for h in hs])
+    for v in kat["fused"]:
+        t = float(bits_to_f32([v["thrd_bits"]])[0])
+        C, R = gpu_quantize(bits_to_f32(v["g_bits"]), t, r_in_np=bits_to_f32(v["r_in_bits"]))
+        assert [f"{w:08X}" for w in C] == v["words"], v["name"]
+        assert_bits_equal(R, nan_bits(v["r_bits"]), v["name"])
     for v in kat["accumulate"]:
         t = float(bits_to_f32([v["thrd_bits"]])[0])
         pl = [dev(np.array([int(h, 16) for h in p], dtype=np.uint32)) for p in v["payload_words"]]
-        acc = torch.full((v["n"],), 3.0, device="cuda")
-        q.cu_fn_dequantize_accumulate_e(acc, pl, t)
-        assert_bits_equal(acc.cpu().numpy(), bits_to_f32(v["acc_bits"]), v["name"])
+        if "acc_in_bits" in v:
+            acc = dev(bits_to_f32(v["acc_in_bits"]))
+            q.cu_fn_dequantize_accumulate_e(acc, pl, t, accumulate=True)
+        else:
+            acc = torch.full((v["n"],), 3.0, device="cuda")
+            q.cu_fn_dequantize_accumulate_e(acc, pl, t)
+        assert_bits_equal(acc.cpu().numpy(), nan_bits(v["acc_bits"]), v["name"])
 
 
 def test_flat_sizes_all_knobs(knobs):
@@ -360,6 +370,51 @@ def test_two_host_threads_on_two_streams():
     for i in range(2):
         assert_words_equal(results[i][0], work[i][2][0], f"thread {i}")
         assert_bits_equal(results[i][1], work[i][2][1], f"thread {i}")
+
+
+def test_one_thread_turns_the_knobs_while_another_launches():
+    """The launch knobs are process-wide atomics and every call works from one snapshot of them:
+    a thread that keeps changing them must not disturb the results (or the launches) of another."""
+    import threading
+    rng = np.random.default_rng(56)
+    n = 1_000_000 + 77
+    g = rng.normal(0, 1e-3, n).astype(np.float32)
+    r = rng.normal(0, 5e-4, n).astype(np.float32)
+    want_c, want_r = oracle.c.quantize(g, 1e-3, R_in=r)
+    want_d = oracle.c.dequantize(want_c, n, 1e-3)
+    old = [_lib.tune(i) for i in range(_lib.N_TUNE)]
+    stop = threading.Event()
+
+    def turn():
+        k = 0
+        while not stop.is_set():
+            k += 1
+            _lib.tune(_lib.TUNE_CHUNKS_PER_WAVE, (1, 2, 4)[k % 3])
+            _lib.tune(_lib.TUNE_WORKGROUP_SIZE, (64, 128, 256, 512, 1024)[k % 5])
+            _lib.tune(_lib.TUNE_NONTEMPORAL, k % 2)
+            _lib.tune(_lib.TUNE_XCD_INTERLEAVE_LOG2, k % 7)
+            _lib.tune(_lib.TUNE_XCD_INTERLEAVE_LOG2_DECODE, (k // 2) % 7)
+            _lib.tune(_lib.TUNE_XCD_INTERLEAVE_LOG2_ACCUMULATE, (k // 3) % 7)
+
+    t = threading.Thread(target=turn)
+    t.start()
+    try:
+        dg, dr0 = dev(g), dev(r)
+        for _ in range(40):
+            dr, dc = dr0.clone(), words_like(n)
+            q.cu_fn_matrix_quantize_e(dg, dc, dr, 1e-3, add_residual=True)
+            assert_words_equal(host_words(dc), want_c)
+            assert_bits_equal(dr.cpu().numpy(), want_r)
+            out = torch.full((n,), 5.0, device="cuda")
+            q.cu_fn_dequantize_accumulate_e(out, [dc, dc], 1e-3)
+            q.cu_fn_matrix_dequantize_e(out, dc, None, 1e-3)
+            assert_bits_equal(out.cpu().numpy(), want_d)
+    finally:
+        stop.set()
+        t.join()
+        for i, v in enumerate(old):
+            _lib.tune(i, v)
+
 
 
 def test_empty_inputs_are_no_ops():

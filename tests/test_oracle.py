@@ -42,16 +42,34 @@ def test_dequantize_kat(kat, name, impl):
         assert_bits_equal(out, bits_to_f32(v["out_bits"]), f"{name}:{v['name']}")
 
 
+def _nan_bits(hexes):
+    return bits_to_f32([("7FC00000" if h == "NAN" else h) for h in hexes])
+
+
+@pytest.mark.parametrize("name,impl", IMPLS)
+def test_fused_kat(kat, name, impl):
+    """Error-feedback step a = fl32(g + r_in), worked by hand: signed zeros, sums that round onto
+    +-t, NaN residual."""
+    for v in kat["fused"]:
+        t = float(bits_to_f32([v["thrd_bits"]])[0])
+        g, r_in = bits_to_f32(v["g_bits"]), bits_to_f32(v["r_in_bits"])
+        with np.errstate(invalid="ignore"):
+            C, R = impl.quantize(g, t, R_in=r_in)
+        assert [f"{w:08X}" for w in C] == v["words"], f"{name}:{v['name']}"
+        assert_bits_equal(R, _nan_bits(v["r_bits"]), f"{name}:{v['name']} residual")
+
+
 @pytest.mark.parametrize("name,impl", IMPLS)
 def test_accumulate_kat(kat, name, impl):
     for v in kat["accumulate"]:
         t = float(bits_to_f32([v["thrd_bits"]])[0])
         pl = [np.array([int(h, 16) for h in p], dtype=np.uint32) for p in v["payload_words"]]
-        out = impl.dequant_accumulate(pl, v["n"], t)
-        assert_bits_equal(out, bits_to_f32(v["acc_bits"]), f"{name}:{v['name']}")
+        start = bits_to_f32(v["acc_in_bits"]) if "acc_in_bits" in v else None
+        out = impl.dequant_accumulate(pl, v["n"], t, acc=None if start is None else start.copy())
+        assert_bits_equal(out, _nan_bits(v["acc_bits"]), f"{name}:{v['name']}")
         # continuing a running sum from memory gives the same bits as one pass
-        half = impl.dequant_accumulate(pl[:2], v["n"], t)
-        out2 = impl.dequant_accumulate(pl[2:], v["n"], t, acc=half)
+        half = impl.dequant_accumulate(pl[:1], v["n"], t, acc=None if start is None else start.copy())
+        out2 = impl.dequant_accumulate(pl[1:], v["n"], t, acc=half)
         assert_bits_equal(out2, out, f"{name}:{v['name']} split")
 
 
