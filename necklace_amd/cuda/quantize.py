@@ -144,10 +144,10 @@ class _Kernel:
 
 cu_knl_matrix_quantize_e = _Kernel(
     "cu_knl_matrix_quantize_e",
-    lambda A, C, R, thrd, stream: _quantize(A, C, R, thrd, False, stream or None, False))
+    lambda A, C, R, thrd, stream: _quantize(A, C, R, thrd, False, stream, False))
 cu_knl_matrix_dequantize_e = _Kernel(
     "cu_knl_matrix_dequantize_e",
-    lambda A, C, R, thrd, stream: _dequantize(A, C, thrd, stream or None, False))
+    lambda A, C, R, thrd, stream: _dequantize(A, C, thrd, stream, False))
 
 
 def cu_fn_matrix_quantize_e(A, C, R, thrd=0.3,
@@ -163,7 +163,7 @@ def cu_fn_matrix_quantize_e(A, C, R, thrd=0.3,
     """
     if to_device:
         A, R, C = _to_device(A), _to_device(R), _to_device(C)
-    _quantize(A, C, R, thrd, add_residual, stream or None, sync)
+    _quantize(A, C, R, thrd, add_residual, stream, sync)
     return (A, C, R) if to_device else None
 
 
@@ -177,7 +177,7 @@ def cu_fn_matrix_dequantize_e(A, C, R, thrd=0.3,
     if to_device:
         A, C = _to_device(A), _to_device(C)
         R = _to_device(R) if R is not None else None
-    _dequantize(A, C, thrd, stream or None, sync)
+    _dequantize(A, C, thrd, stream, sync)
     return (A, C, R) if to_device else None
 
 

@@ -117,26 +117,24 @@ class GradCompressor:
                 self.grd_resi.append(None)
                 self.grd_comp.append(None)
                 self.grd_recv.append(None)
-        # argument tables of the many-vectors entry points; everything but the gradients' own
-        # addresses is fixed for the life of the buffers
+        # argument tables of the many-vectors entry points: everything but the gradients' own
+        # addresses is fixed for the life of the buffers (built on first use, per subset of
+        # parameters that have a gradient)
         self._idx = [i for i, c in enumerate(self.grd_cmps) if c]
-        m = len(self._idx)
-        self._n_arr = (ct.c_uint64 * m)(*[lay.numels[i] for i in self._idx])
-        self._wo_arr = (ct.c_uint64 * m)(*[lay.word_offset[i] for i in self._idx])
-        self._r_arr = (ct.c_void_p * m)(*[self.grd_resi[i].data_ptr() for i in self._idx])
-        self._c_arr = (ct.c_void_p * m)(*[self.grd_comp[i].data_ptr() for i in self._idx])
+        self._live_key, self._live_tabs = None, None
         self._pl_arr = (ct.c_void_p * self.kn)(*[self.recv[k].data_ptr() for k in range(self.kn)])
 
-    def _ptrs(self, tensors, what):
-        """Device addresses of the compressed parameters' tensors, after checking them."""
+    def _tables(self, tensors, what):
+        """Argument tables for the compressed parameters whose tensor is present (not None) in this
+        call; cached while the same subset comes back.  Returns (count, ptrs, r, c, n, word_offset)."""
         if len(tensors) != len(self.layout):
             raise ValueError(f"expected {len(self.layout)} {what}s, got {len(tensors)}")
-        for i in self._idx:
+        live = [i for i in self._idx if tensors[i] is not None]
+        for i in live:
             if tensors[i].numel() != self.layout.numels[i]:
                 raise ValueError(
                     f"{what} {i}: {tensors[i].numel()} elements, layout has {self.layout.numels[i]}")
-        out = []
-        for i in self._idx:
+        for i in live:
             t = tensors[i]
             if t.dtype != torch.float32 or not t.is_cuda:
                 raise TypeError(f"{what} {i}: expected a float32 GPU tensor, got {t.dtype} on {t.device}")
@@ -144,24 +142,33 @@ class GradCompressor:
                 raise ValueError(f"{what} {i} must be contiguous")
             if t.device != self.resi.device:
                 raise ValueError(f"{what} {i} is on {t.device}, the buffers are on {self.resi.device}")
-            out.append(t.data_ptr())
-        return (ct.c_void_p * len(out))(*out)
+        key = tuple(live)
+        if key != self._live_key:
+            m = len(live)
+            self._live_key = key
+            self._live_tabs = (
+                (ct.c_void_p * m)(*[self.grd_resi[i].data_ptr() for i in live]),
+                (ct.c_void_p * m)(*[self.grd_comp[i].data_ptr() for i in live]),
+                (ct.c_uint64 * m)(*[self.layout.numels[i] for i in live]),
+                (ct.c_uint64 * m)(*[self.layout.word_offset[i] for i in live]))
+        ptrs = (ct.c_void_p * len(live))(*[tensors[i].data_ptr() for i in live])
+        return (len(live), ptrs) + self._live_tabs
 
     # ---- send side
 
     def compress(self, grads, stream=None, sync=False):
         """Quantize every compressed parameter's gradient with error feedback.
 
-        `grads[i]` is parameter i's gradient (any shape, contiguous fp32 on the GPU);
-        entries of uncompressed parameters are ignored.  One launch per 96 parameters.
+        `grads[i]` is parameter i's gradient (any shape, contiguous fp32 on the GPU), or None when
+        the parameter has no gradient this step (its residual and code words are left as they
+        are); entries of uncompressed parameters are ignored.  One launch per 96 parameters.
         """
-        g_arr = self._ptrs(grads, "gradient")
-        if not self._idx:
+        m, g_arr, r_arr, c_arr, n_arr, _ = self._tables(grads, "gradient")
+        if not m:
             return
         with torch.cuda.device(self.resi.device):
             _lib.check(_lib.lib().nklq_quantize_multi_f32(
-                len(self._idx), g_arr, self._r_arr, self._c_arr, self._n_arr, self.thrd, 1,
-                _nb.stream_handle(stream, self.resi.device)))
+                m, g_arr, r_arr, c_arr, n_arr, self.thrd, 1, _nb.stream_handle(stream, self.resi.device)))
         if sync:
             _sync(self.device, stream)
 
@@ -184,13 +191,14 @@ class GradCompressor:
 
     def decompress_sum(self, outs, average=True, stream=None, sync=False):
         """outs[i] <- sum over ranks k = 0..kn-1 (in that order) of decode(recv[k] of parameter i),
-        divided by kn when `average` (the `/ kn` of necklace/frmwrk/pytorch/ptprms.py:294)."""
-        o_arr = self._ptrs(outs, "output")
-        if not self._idx:
+        divided by kn when `average` (the `/ kn` of necklace/frmwrk/pytorch/ptprms.py:294).
+        Entries that are None are skipped, as in `compress`."""
+        m, o_arr, _, _, n_arr, wo_arr = self._tables(outs, "output")
+        if not m:
             return
         with torch.cuda.device(self.resi.device):
             _lib.check(_lib.lib().nklq_dequant_accumulate_multi_f32(
-                len(self._idx), o_arr, self._n_arr, self._wo_arr, self._pl_arr, self.kn, self.thrd, 0,
+                m, o_arr, n_arr, wo_arr, self._pl_arr, self.kn, self.thrd, 0,
                 float(self.kn) if average else 1.0, _nb.stream_handle(stream, self.resi.device)))
         if sync:
             _sync(self.device, stream)
@@ -253,25 +261,45 @@ def init_grad_comp_cfg(params, kn, grad_comp_cfg=None, device="cuda", rank=0):
     return cfg
 
 
+def _run_exchange(exchange, gc, kn, stream):
+    """Calls the caller's all-gather of the payloads in stream order with the kernels around it.
+
+    The kernels run on `stream` (None: torch's current stream); `exchange(comp, recv)` is called
+    with torch's current stream as it is, which is where a collective issued through torch runs.
+    When the two differ, the current stream first waits for the compress, and `stream` then waits
+    for what the exchange put on the current stream."""
+    if exchange is None:
+        if kn != 1:
+            raise ValueError("an exchange callable is required when kn > 1")
+        return
+    cur = torch.cuda.current_stream(gc.device)
+    other = stream is not None and not isinstance(stream, int) and stream != cur
+    if isinstance(stream, int) and stream != cur.cuda_stream:
+        raise ValueError("with a raw stream handle the exchange cannot be ordered: pass a torch.cuda.Stream")
+    if other:
+        cur.wait_stream(stream)
+    exchange(gc.comp, gc.recv)
+    if other:
+        stream.wait_stream(cur)
+
+
 def grads_do_compressed_exchange(grads, kn, grad_comp_cfg, exchange=None, average=True, stream=None):
     """The compressed form of the gradient all-reduce (what ``grads_do_nccl(..., grad_comp_cfg=)``
     stands for at necklace/trainer/tnopmx.py:334-337): compress, exchange, decompress-sum in place.
 
     `exchange(comp, recv)` must fill ``recv[k]`` with rank k's payload for all k (an all-gather of
     `comp`); it is the caller's, since collectives are not part of this module.  With ``kn == 1``
-    it may be omitted.  Returns the indices of the parameters that were NOT compressed and still
-    need the ordinary fp32 all-reduce.
+    it may be omitted.  Entries of `grads` may be None (no gradient this step).  Returns the
+    indices of the parameters that were NOT compressed (below the size threshold) and still need
+    the ordinary fp32 all-reduce.
     """
     gc = grad_comp_cfg["compressor"]
     if gc.kn != kn:
         raise ValueError(f"grad_comp_cfg was built for kn={gc.kn}, got kn={kn}")
     gc.compress(grads, stream=stream)
-    if exchange is not None:
-        exchange(gc.comp, gc.recv)
-    elif kn != 1:
-        raise ValueError("an exchange callable is required when kn > 1")
+    _run_exchange(exchange, gc, kn, stream)
     gc.decompress_sum(grads, average=average, stream=stream)
-    return [i for i, c in enumerate(gc.grd_cmps) if not c]
+    return [i for i, c in enumerate(gc.grd_cmps) if not c and grads[i] is not None]
 
 
 # --------------------------------------------------------------------------- flat gradient buffer
@@ -286,23 +314,27 @@ def init_flat_grad_comp_cfg(total_size, kn, grad_comp_cfg=None, device="cuda", r
     return init_grad_comp_cfg([int(total_size)], kn, cfg, device=device, rank=rank)
 
 
+def _flat_view(d_arr_send, sz):
+    if not d_arr_send.is_contiguous():
+        raise ValueError("the flat gradient buffer must be contiguous (the result is written in place)")
+    return d_arr_send.view(-1)[:sz]
+
+
 def opt_grads_fltn_do_compressed_reduce(kn, d_arr_send, sz, grad_comp_cfg, exchange=None, average=False,
-                                        stream=None):
+                                        stream=None, decode=True):
     """Compressed form of ``opt_grads_fltn_do_nccl_reduce(nc, kn, root, d_arr_send, sz, grad_comp_cfg)``
     (necklace/frmwrk/pytorch/ptprms.py:396-401): the first `sz` floats of the flat buffer
     `d_arr_send` are quantized with error feedback (one launch per 2^28 elements), `exchange(comp,
-    recv)` gathers every rank's payload, and the decoded sum over ranks, in rank order, replaces
-    them.  The reference's reduce does not average; pass ``average=True`` for ``/ kn``."""
+    recv)` gathers every rank's payload, and (with `decode`) the decoded sum over ranks, in rank
+    order, replaces them.  The reference's reduce does not average; pass ``average=True`` for ``/ kn``."""
     gc = grad_comp_cfg["compressor"]
     if gc.kn != kn:
         raise ValueError(f"grad_comp_cfg was built for kn={gc.kn}, got kn={kn}")
-    flat = d_arr_send.reshape(-1)[:sz]
+    flat = _flat_view(d_arr_send, sz)
     gc.compress_flat(flat, stream=stream)
-    if exchange is not None:
-        exchange(gc.comp, gc.recv)
-    elif kn != 1:
-        raise ValueError("an exchange callable is required when kn > 1")
-    gc.decompress_sum([flat], average=average, stream=stream)
+    _run_exchange(exchange, gc, kn, stream)
+    if decode:
+        gc.decompress_sum([flat], average=average, stream=stream)
 
 
 # --------------------------------------------------------------------------- checkpoint
@@ -324,86 +356,205 @@ def load_grad_comp_state(grad_comp_cfg, state):
 
 
 # --------------------------------------------------------------------------- ptprms call surface
+#
+# Same names, argument order and return value (None) as necklace/frmwrk/pytorch/ptprms.py:319-401, so
+# that a trainer can import them from here instead.  What differs is what travels:
+#
+#   nc             where necklace passes its NCCL communicator.  Collectives are not part of this
+#                  package, so `nc` is whatever moves the data: a callable ``nc(comp, recv)`` that
+#                  all-gathers the packed words, or an object with ``all_gather_words(comp, recv)``
+#                  and, for the gradients that stay fp32, ``all_reduce_f32(flat)`` /
+#                  ``reduce_f32(flat, root)`` (sum, in place).  None is allowed for kn == 1.
+#   grad_comp_cfg  the dict of necklace/trainer/tnopmx.py:135-151 (grad_size_threshold,
+#                  grad_comp_threshold) plus: 'rank' (this worker), 'form' ("params": every gradient
+#                  of at least grad_size_threshold elements is packed on its own, the smaller ones
+#                  are flattened into one fp32 message, the default; "buckets": all gradients are
+#                  flattened into buckets of at most 'bucket_bytes' = 256 MB and each bucket is packed
+#                  as one vector, the shape of nccl_allreduce_by_buckets, ptprms.py:256-299),
+#                  'small_allreduce' / 'small_reduce' (callables that override nc's fp32 methods).
+#                  The buffers are laid out on the first call and kept in the dict.
+#   prm_revs       accepted and unused, as in the reference.
 
-def _opt_grads(opt):
-    """The gradients an optimizer owns, in the order necklace walks them
+NCCL_REDUCE_BUCKET_BYTES = 256 * 1024 * 1024  # nccl_reduce_bucket_size, necklace/frmwrk/pytorch/ptprms.py:253
+
+
+def _opt_params(opt):
+    """Every parameter an optimizer owns, in the order necklace walks them
     (necklace/frmwrk/pytorch/ptprms.py:331-336)."""
-    grads = []
-    for group in opt.param_groups:
-        for p in group["params"]:
-            if p.grad is not None:
-                grads.append(p.grad.data)
-    return grads
+    return [p for group in opt.param_groups for p in group["params"]]
 
 
 def _exchange_of(nc):
-    """`nc` stands where necklace passes its NCCL communicator.  Collectives are not part of this
-    package, so it is whatever gathers the payloads: a callable ``nc(comp, recv)`` or an object
-    with ``all_gather_words(comp, recv)``; None is allowed for a single worker."""
-    if nc is None or callable(nc):
+    if nc is None or (callable(nc) and not hasattr(nc, "all_gather_words")):
         return nc
     return nc.all_gather_words
 
 
-def _cfg_for(grads, kn, grad_comp_cfg):
+def _small_fn(nc, cfg, root):
+    """The fp32 collective for what is not compressed: sums `flat` over the workers in place."""
+    key, meth = ("small_allreduce", "all_reduce_f32") if root is None else ("small_reduce", "reduce_f32")
+    fn = cfg.get(key) or getattr(nc, meth, None)
+    if fn is None:
+        return None
+    return fn if root is None else (lambda flat: fn(flat, root))
+
+
+def _take_buckets(tensors, limit_bytes):
+    """Consecutive groups of tensors of at most `limit_bytes` each (a tensor larger than that is a
+    group of its own): the bucketing of ptprms.py:258 for tensors of one type."""
+    buckets, cur, size = [], [], 0
+    for t in tensors:
+        b = t.numel() * t.element_size()
+        if cur and size + b > limit_bytes:
+            buckets.append(cur)
+            cur, size = [], 0
+        cur.append(t)
+        size += b
+    if cur:
+        buckets.append(cur)
+    return buckets
+
+
+def _carry_residuals(old_gc, old_ids, new_gc, new_ids):
+    """Error feedback owed to a parameter survives a change of the layout."""
+    if old_gc is None:
+        return
+    where = {pid: i for i, pid in enumerate(old_ids)}
+    for j, pid in enumerate(new_ids):
+        i = where.get(pid)
+        if i is not None and old_gc.grd_resi[i] is not None and new_gc.grd_resi[j] is not None \
+                and old_gc.grd_resi[i].numel() == new_gc.grd_resi[j].numel():
+            new_gc.grd_resi[j].copy_(old_gc.grd_resi[i])
+
+
+def _cfg_for_params(params, kn, cfg):
+    """Lay the buffers out over ALL parameters of the optimizer (a parameter without a gradient is
+    skipped per call); rebuilt, residuals carried over, when the optimizer's parameters change."""
+    ids = [id(p) for p in params]
+    sig = ("params", tuple((i, p.numel()) for i, p in zip(ids, params)), kn)
+    if cfg.get("_signature") != sig:
+        old_gc, old_ids = cfg.get("compressor"), cfg.get("_ids", [])
+        dev = next((p.device for p in params if p.is_cuda), torch.device("cuda"))
+        built = init_grad_comp_cfg(params, kn, cfg, device=dev, rank=cfg.get("rank", 0))
+        _carry_residuals(old_gc if cfg.get("_signature", ("",))[0] == "params" else None, old_ids,
+                         built["compressor"], ids)
+        cfg.update(built)
+        cfg["_signature"], cfg["_ids"] = sig, ids
+    return cfg["compressor"]
+
+
+def _reduce_small(small, kn, fn, average):
+    """The gradients below the size threshold, as ONE flattened fp32 message
+    (flatten -> collective -> / kn -> copy back, ptprms.py:261-299)."""
+    if not small:
+        return
+    if kn == 1:
+        return  # the sum over one worker, divided by one
+    if fn is None:
+        raise ValueError(
+            f"{len(small)} gradients are below grad_size_threshold and kn > 1: give nc an all_reduce_f32 / "
+            "reduce_f32 method or put 'small_allreduce' / 'small_reduce' into grad_comp_cfg")
+    flat = torch.cat([g.reshape(-1) for g in small])
+    fn(flat)
+    if average:
+        flat /= float(kn)
+    pos = 0
+    for g in small:
+        g.copy_(flat[pos:pos + g.numel()].view_as(g))
+        pos += g.numel()
+
+
+def _reduce_params_form(nc, kn, root, params, cfg):
+    gc = _cfg_for_params(params, kn, cfg)
+    grads = [p.grad.data if p.grad is not None else None for p in params]
+    if all(g is None for g in grads):
+        return
+    average = root is None  # the reference's reduce leaves `/ kn` commented out (ptprms.py:385)
+    gc.compress(grads)
+    _run_exchange(_exchange_of(nc), gc, kn, None)
+    if root is None or gc.rank == root:
+        gc.decompress_sum(grads, average=average)
+    small = [g for g, c in zip(grads, gc.grd_cmps) if g is not None and not c]
+    _reduce_small(small, kn, _small_fn(nc, cfg, root), average)
+
+
+def _reduce_buckets_form(nc, kn, root, params, cfg):
+    grads = [p.grad.data for p in params if p.grad is not None]
+    if not grads:
+        return
+    buckets = _take_buckets(grads, int(cfg.get("bucket_bytes", NCCL_REDUCE_BUCKET_BYTES)))
+    sizes = [sum(g.numel() for g in b) for b in buckets]
+    sig = ("buckets", tuple(tuple(g.numel() for g in b) for b in buckets), kn)
+    if cfg.get("_signature") != sig:
+        sub = dict(cfg)
+        sub["grad_size_threshold"] = 1  # a bucket is always packed
+        built = init_grad_comp_cfg(sizes, kn, sub, device=grads[0].device, rank=cfg.get("rank", 0))
+        for key in ("grd_resi", "grd_recv", "grd_comp", "grd_cmps", "compressor"):
+            cfg[key] = built[key]
+        cfg["_signature"] = sig
+        cfg["_flat"] = [torch.empty(n, dtype=torch.float32, device=grads[0].device) for n in sizes]
+    gc, flats = cfg["compressor"], cfg["_flat"]
+    for flat, bucket in zip(flats, buckets):  # grads_batch_coalesced, ptprms.py:262
+        torch.cat([g.reshape(-1) for g in bucket], out=flat)
+    gc.compress(flats)
+    _run_exchange(_exchange_of(nc), gc, kn, None)
+    if root is None or gc.rank == root:
+        gc.decompress_sum(flats, average=root is None)
+        for flat, bucket in zip(flats, buckets):  # unflatten and copy back, ptprms.py:296-299
+            pos = 0
+            for g in bucket:
+                g.copy_(flat[pos:pos + g.numel()].view_as(g))
+                pos += g.numel()
+
+
+def _reduce_opt(nc, kn, root, opt, grad_comp_cfg):
     if grad_comp_cfg is None:
         raise ValueError("grad_comp_cfg is required: this is the compressed path")
-    if "compressor" not in grad_comp_cfg:
-        # first call: lay the buffers out for these gradients (trainer/tnopmx.py:135-151 does this
-        # once at set-up; doing it lazily here keeps the call sites of ptprms unchanged)
-        built = init_grad_comp_cfg(grads, kn, grad_comp_cfg, device=grads[0].device,
-                                   rank=grad_comp_cfg.get("rank", 0))
-        grad_comp_cfg.update(built)
-    return grad_comp_cfg
+    params = _opt_params(opt)
+    form = grad_comp_cfg.get("form", "params")
+    if form == "params":
+        _reduce_params_form(nc, kn, root, params, grad_comp_cfg)
+    elif form == "buckets":
+        _reduce_buckets_form(nc, kn, root, params, grad_comp_cfg)
+    else:
+        raise ValueError(f"grad_comp_cfg['form'] must be 'params' or 'buckets', got {form!r}")
+
+
+def _per_optimizer(opt, grad_comp_cfg):
+    if not isinstance(opt, (list, tuple)):
+        return [(opt, grad_comp_cfg)]
+    if len(opt) > 1 and not isinstance(grad_comp_cfg, (list, tuple)):
+        raise ValueError("several optimizers need one grad_comp_cfg each (their residuals differ)")
+    cfgs = grad_comp_cfg if isinstance(grad_comp_cfg, (list, tuple)) else [grad_comp_cfg] * len(opt)
+    return list(zip(opt, cfgs))
 
 
 def opt_one_grads_do_nccl_allreduce(nc, kn, opt, prm_revs=None, grad_comp_cfg=None):
     """Compressed counterpart of ptprms.opt_one_grads_do_nccl_allreduce
-    (necklace/frmwrk/pytorch/ptprms.py:329-338): every gradient of at least
-    ``grad_size_threshold`` elements is replaced by the average over the `kn` workers of its 2-bit
-    decode.  Returns the gradients below the threshold: they still need the ordinary all-reduce."""
-    grads = _opt_grads(opt)
-    if not grads:
-        return []
-    cfg = _cfg_for(grads, kn, grad_comp_cfg)
-    small = grads_do_compressed_exchange(grads, kn, cfg, exchange=_exchange_of(nc), average=True)
-    return [grads[i] for i in small]
+    (necklace/frmwrk/pytorch/ptprms.py:329-338): afterwards EVERY gradient of the optimizer holds
+    the average over the `kn` workers — of its 2-bit decode where it was packed, of its fp32 values
+    where it was too small to pack.  Returns None, like the reference."""
+    _reduce_opt(nc, kn, None, opt, grad_comp_cfg)
 
 
 def opt_grads_do_nccl_allreduce(nc, kn, opt, prm_revs=None, grad_comp_cfg=None):
     """ptprms.opt_grads_do_nccl_allreduce (ptprms.py:319-326): one optimizer or a list of them, each
-    with its own ``grad_comp_cfg`` entry when a list of configs is given."""
-    if isinstance(opt, (list, tuple)):
-        cfgs = grad_comp_cfg if isinstance(grad_comp_cfg, (list, tuple)) else [grad_comp_cfg] * len(opt)
-        if len(opt) > 1 and not isinstance(grad_comp_cfg, (list, tuple)):
-            raise ValueError("several optimizers need one grad_comp_cfg each (their residuals differ)")
-        out = []
-        for o, c in zip(opt, cfgs):
-            out += opt_one_grads_do_nccl_allreduce(nc, kn, o, prm_revs=prm_revs, grad_comp_cfg=c)
-        return out
-    return opt_one_grads_do_nccl_allreduce(nc, kn, opt, prm_revs=prm_revs, grad_comp_cfg=grad_comp_cfg)
+    with its own ``grad_comp_cfg`` when a list of configs is given."""
+    for o, c in _per_optimizer(opt, grad_comp_cfg):
+        opt_one_grads_do_nccl_allreduce(nc, kn, o, prm_revs=prm_revs, grad_comp_cfg=c)
+
+
+def opt_one_grads_do_nccl_reduce(nc, kn, root, opt, prm_revs=None, grad_comp_cfg=None):
+    """Compressed counterpart of ptprms.opt_one_grads_do_nccl_reduce (ptprms.py:354-363): like the
+    all-reduce but only worker `root` ends up with the sums, and they are not averaged (the
+    reference's reduce leaves the `/ kn` commented out, ptprms.py:385).  Returns None."""
+    _reduce_opt(nc, kn, root, opt, grad_comp_cfg)
 
 
 def opt_grads_do_nccl_reduce(nc, kn, root, opt, prm_revs=None, grad_comp_cfg=None):
-    """Compressed counterpart of ptprms.opt_grads_do_nccl_reduce (ptprms.py:344-363): like the
-    all-reduce but only worker `root` decodes, and the sum is not averaged (the reference's reduce
-    leaves the `/ kn` commented out, ptprms.py:385)."""
-    grads = _opt_grads(opt)
-    if not grads:
-        return []
-    cfg = _cfg_for(grads, kn, grad_comp_cfg)
-    gc = cfg["compressor"]
-    if gc.kn != kn:
-        raise ValueError(f"grad_comp_cfg was built for kn={gc.kn}, got kn={kn}")
-    gc.compress(grads)
-    exchange = _exchange_of(nc)
-    if exchange is not None:
-        exchange(gc.comp, gc.recv)
-    elif kn != 1:
-        raise ValueError("an exchange is required when kn > 1")
-    if gc.rank == root:
-        gc.decompress_sum(grads, average=False)
-    return [grads[i] for i, c in enumerate(gc.grd_cmps) if not c]
+    """ptprms.opt_grads_do_nccl_reduce (ptprms.py:344-351)."""
+    for o, c in _per_optimizer(opt, grad_comp_cfg):
+        opt_one_grads_do_nccl_reduce(nc, kn, root, o, prm_revs=prm_revs, grad_comp_cfg=c)
 
 
 def opt_grads_fltn_do_nccl_reduce(nc, kn, root, d_arr_send, sz, grad_comp_cfg=None):
@@ -412,14 +563,5 @@ def opt_grads_fltn_do_nccl_reduce(nc, kn, root, d_arr_send, sz, grad_comp_cfg=No
     if grad_comp_cfg is None or "compressor" not in grad_comp_cfg:
         raise ValueError("build grad_comp_cfg with init_flat_grad_comp_cfg first")
     gc = grad_comp_cfg["compressor"]
-    if gc.kn != kn:
-        raise ValueError(f"grad_comp_cfg was built for kn={gc.kn}, got kn={kn}")
-    flat = d_arr_send.reshape(-1)[:sz]
-    gc.compress_flat(flat)
-    exchange = _exchange_of(nc)
-    if exchange is not None:
-        exchange(gc.comp, gc.recv)
-    elif kn != 1:
-        raise ValueError("an exchange is required when kn > 1")
-    if gc.rank == root:
-        gc.decompress_sum([flat], average=False)
+    opt_grads_fltn_do_compressed_reduce(kn, d_arr_send, sz, grad_comp_cfg, exchange=_exchange_of(nc),
+                                        average=False, decode=gc.rank == root)

@@ -141,47 +141,165 @@ def test_checkpoint_file_round_trip(tmp_path):
     assert state["epoch"] == 3
 
 
-def test_ptprms_call_surface_on_a_real_optimizer():
-    """opt_grads_do_nccl_allreduce / _reduce with necklace's argument order on the gradients of a
-    small MLP (the shape of the reference's MNIST example), two workers whose payloads coincide."""
-    torch.manual_seed(0)
+class TwoWorkersWithEqualData:
+    """Stands where necklace passes its NCCL communicator: a second worker that holds exactly what
+    this one holds (so every sum is x + x), with the three collectives the compressed path needs."""
+    def __init__(self, rank=0):
+        self.calls, self.rank = [], rank
+
+    def all_gather_words(self, comp, recv):
+        self.calls.append(("gather", comp.numel()))
+        recv[1 - self.rank].copy_(recv[self.rank])
+
+    def all_reduce_f32(self, flat):
+        self.calls.append(("allreduce", flat.numel()))
+        flat.mul_(2.0)
+
+    def reduce_f32(self, flat, root):
+        self.calls.append(("reduce", flat.numel(), root))
+        flat.mul_(2.0)
+
+
+def _mlp_with_grads(seed=0):
+    torch.manual_seed(seed)
     model = torch.nn.Sequential(torch.nn.Linear(784, 256), torch.nn.ReLU(), torch.nn.Linear(256, 64),
                                 torch.nn.ReLU(), torch.nn.Linear(64, 10)).cuda()
     opt = torch.optim.SGD(model.parameters(), lr=0.1)
     x = torch.randn(32, 784, device="cuda")
-    loss = torch.nn.functional.cross_entropy(model(x), torch.randint(0, 10, (32,), device="cuda"))
-    loss.backward()
+    y = torch.randint(0, 10, (32,), device="cuda")
+    torch.nn.functional.cross_entropy(model(x), y).backward()
+    return model, opt, x, y
+
+
+def test_ptprms_call_surface_on_a_real_optimizer():
+    """opt_grads_do_nccl_allreduce / _reduce with necklace's argument order on the gradients of a
+    small MLP (the shape of the reference's MNIST example).  Like the reference functions
+    (necklace/frmwrk/pytorch/ptprms.py:319-363) they return None and leave EVERY gradient reduced:
+    the large ones through the 2-bit codes, the small ones as one flattened fp32 message."""
+    model, opt, x, y = _mlp_with_grads()
     thrd, kn = 1e-3, 2
     before = [p.grad.detach().cpu().numpy().copy() for p in model.parameters()]
-
-    def same_payload_from_both(comp, recv):
-        recv[1].copy_(recv[0])
-
+    nc = TwoWorkersWithEqualData()
     cfg = {"grad_comp_threshold": thrd, "grad_size_threshold": 1001}
-    small = ptcomp.opt_grads_do_nccl_allreduce(same_payload_from_both, kn, opt, None, grad_comp_cfg=cfg)
+    assert ptcomp.opt_grads_do_nccl_allreduce(nc, kn, opt, None, grad_comp_cfg=cfg) is None
     torch.cuda.synchronize()
     assert "compressor" in cfg
-    sizes = [g.size for g in before]
-    assert sorted(t.numel() for t in small) == sorted(s for s in sizes if s < 1001)
+    n_small = sum(g.size for g in before if g.size < 1001)
+    assert ("allreduce", n_small) in nc.calls and nc.calls[0][0] == "gather"
     for p, g in zip(model.parameters(), before):
         got = p.grad.detach().cpu().numpy()
         if g.size < 1001:
-            assert_bits_equal(got, g, "small gradients are left to the ordinary all-reduce")
+            want = ((g + g) / np.float32(kn)).astype(np.float32)  # fp32 sum of two equal workers, averaged
+            assert_bits_equal(got, want, "small gradients are averaged in fp32")
             continue
         c, _ = oracle.c.quantize(g.reshape(-1), thrd, R_in=np.zeros(g.size, np.float32))
         want = (oracle.c.dequant_accumulate([c, c], g.size, thrd) / np.float32(kn)).astype(np.float32)
         assert_bits_equal(got.reshape(-1), want, f"gradient of {g.shape}")
-    # reduce-to-root: the non-root worker compresses and sends but keeps its gradient
+    # without a way to reduce the small gradients the call refuses instead of skipping them
+    with pytest.raises(ValueError):
+        ptcomp.opt_grads_do_nccl_allreduce(lambda comp, recv: None, kn, opt, None,
+                                           grad_comp_cfg={"grad_comp_threshold": thrd})
+    # reduce-to-root: the non-root worker compresses and sends but keeps its large gradients
     cfg1 = {"grad_comp_threshold": thrd, "rank": 1}
-    loss = torch.nn.functional.cross_entropy(model(x), torch.randint(0, 10, (32,), device="cuda"))
     opt.zero_grad(set_to_none=False)
-    loss.backward()
+    torch.nn.functional.cross_entropy(model(x), y).backward()
     keep = [p.grad.detach().clone() for p in model.parameters()]
-    ptcomp.opt_grads_do_nccl_reduce(lambda comp, recv: None, kn, 0, opt, None, grad_comp_cfg=cfg1)
+    nc1 = TwoWorkersWithEqualData(rank=1)
+    assert ptcomp.opt_grads_do_nccl_reduce(nc1, kn, 0, opt, None, grad_comp_cfg=cfg1) is None
     torch.cuda.synchronize()
     for p, k in zip(model.parameters(), keep):
-        assert torch.equal(p.grad, k)
+        if p.numel() >= 1001:
+            assert torch.equal(p.grad, k)
+        else:
+            assert torch.equal(p.grad, k * 2.0)  # summed by nc.reduce_f32, not averaged (ptprms.py:385)
+    assert ("reduce", n_small, 0) in nc1.calls
     assert int((cfg1["compressor"].comp != 0).sum()) > 0
+
+
+def test_a_gradient_that_first_appears_at_step_two_and_a_parameter_added_later():
+    """The layout covers all parameters of the optimizer from the start, so one whose .grad is None
+    at step 1 simply joins at step 2 with a zero residual; a parameter group added later rebuilds
+    the layout and carries the residuals over."""
+    torch.manual_seed(3)
+    thrd = 1e-3
+    a = torch.nn.Parameter(torch.randn(3000, device="cuda") * 1e-3)
+    b = torch.nn.Parameter(torch.randn(5000, device="cuda") * 1e-3)
+    opt = torch.optim.SGD([a, b], lr=0.1)
+    cfg = {"grad_comp_threshold": thrd, "grad_size_threshold": 1}
+    rng = np.random.default_rng(12)
+    ra, rb = np.zeros(3000, np.float32), np.zeros(5000, np.float32)
+
+    def step(ga, gb, gc_=None):
+        a.grad = None if ga is None else dev(ga)
+        b.grad = None if gb is None else dev(gb)
+        ptcomp.opt_grads_do_nccl_allreduce(None, 1, opt, None, grad_comp_cfg=cfg)
+        torch.cuda.synchronize()
+
+    g1 = rng.normal(0, 2e-3, 3000).astype(np.float32)
+    step(g1, None)                                   # step 1: b has no gradient yet
+    c, ra = oracle.c.quantize(g1, thrd, R_in=ra)
+    assert_bits_equal(a.grad.cpu().numpy(), oracle.c.dequantize(c, 3000, thrd), "step 1 a")
+    g2a, g2b = rng.normal(0, 2e-3, 3000).astype(np.float32), rng.normal(0, 2e-3, 5000).astype(np.float32)
+    step(g2a, g2b)                                   # step 2: b joins
+    c, ra = oracle.c.quantize(g2a, thrd, R_in=ra)
+    assert_bits_equal(a.grad.cpu().numpy(), oracle.c.dequantize(c, 3000, thrd), "step 2 a")
+    c, rb = oracle.c.quantize(g2b, thrd, R_in=rb)
+    assert_bits_equal(b.grad.cpu().numpy(), oracle.c.dequantize(c, 5000, thrd), "step 2 b")
+    # step 3: a third parameter enters the optimizer; a and b keep what they are owed
+    d = torch.nn.Parameter(torch.zeros(2000, device="cuda"))
+    opt.add_param_group({"params": [d]})
+    g3a, g3b, g3d = (rng.normal(0, 2e-3, k).astype(np.float32) for k in (3000, 5000, 2000))
+    d.grad = dev(g3d)
+    step(g3a, g3b)
+    c, ra = oracle.c.quantize(g3a, thrd, R_in=ra)
+    assert_bits_equal(a.grad.cpu().numpy(), oracle.c.dequantize(c, 3000, thrd), "step 3 a")
+    c, rb = oracle.c.quantize(g3b, thrd, R_in=rb)
+    assert_bits_equal(b.grad.cpu().numpy(), oracle.c.dequantize(c, 5000, thrd), "step 3 b")
+    c, _ = oracle.c.quantize(g3d, thrd, R_in=np.zeros(2000, np.float32))
+    assert_bits_equal(d.grad.cpu().numpy(), oracle.c.dequantize(c, 2000, thrd), "step 3 d")
+
+
+def test_bucket_form_packs_flattened_buckets_like_nccl_allreduce_by_buckets():
+    """grad_comp_cfg['form'] = 'buckets': gradients are flattened into buckets (here of at most
+    512 KB so that the MLP gives several), every bucket is packed as ONE flat vector, exchanged,
+    decoded, averaged and copied back (necklace/frmwrk/pytorch/ptprms.py:256-299); two steps with
+    the residual carried per bucket."""
+    model, opt, x, y = _mlp_with_grads(seed=5)
+    thrd, kn = 1e-3, 2
+    cfg = {"grad_comp_threshold": thrd, "form": "buckets", "bucket_bytes": 1 << 19}
+    nc = TwoWorkersWithEqualData()
+    resid = None
+    for step in range(2):
+        if step:
+            opt.zero_grad(set_to_none=False)
+            torch.nn.functional.cross_entropy(model(x), y).backward()
+        grads = [p.grad.detach().cpu().numpy().reshape(-1).copy() for p in model.parameters()]
+        assert ptcomp.opt_grads_do_nccl_allreduce(nc, kn, opt, None, grad_comp_cfg=cfg) is None
+        torch.cuda.synchronize()
+        # the same bucketing on the host: consecutive tensors, at most 512 KB per bucket
+        buckets, cur, size = [], [], 0
+        for g in grads:
+            if cur and size + 4 * g.size > (1 << 19):
+                buckets.append(cur)
+                cur, size = [], 0
+            cur.append(g)
+            size += 4 * g.size
+        buckets.append(cur)
+        assert len(buckets) >= 2
+        if resid is None:
+            resid = [np.zeros(sum(g.size for g in b), np.float32) for b in buckets]
+        got = [p.grad.detach().cpu().numpy().reshape(-1) for p in model.parameters()]
+        k = 0
+        for bi, b in enumerate(buckets):
+            flat = np.concatenate(b)
+            c, resid[bi] = oracle.c.quantize(flat, thrd, R_in=resid[bi])
+            want = (oracle.c.dequant_accumulate([c, c], flat.size, thrd) / np.float32(kn)).astype(np.float32)
+            pos = 0
+            for g in b:
+                assert_bits_equal(got[k], want[pos:pos + g.size], f"step {step} bucket {bi} tensor {k}")
+                pos += g.size
+                k += 1
+    assert all(c[0] == "gather" for c in nc.calls)  # nothing stays fp32 in this form
 
 
 def test_sgd_with_compressed_gradients_still_learns():
