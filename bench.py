@@ -13,7 +13,10 @@ fp32 elements, inputs resident in HBM.  Prints one JSON line:
                events on the launch stream, against the 8 TB/s HBM peak
   cpu_baseline the C restatement of the reference kernel (oracle/), OpenMP over
                the host cores, timed on a slab of the same gradient
-  extras       decode (elements/s), 8-payload fixed-order sum, plain copy
+  extras       decode (elements/s), 8-payload fixed-order sum, plain copy, the other four
+               synthetic workloads (config1, config2, config3, config5: kernel time, GB/s of
+               algorithmic bytes, fraction of the HBM peak), wall time per call of the
+               reference-named wrapper at small sizes
 
 The CPU checker is used for the cpu_baseline leg only, never for the GPU path.
 """
@@ -45,9 +48,9 @@ def parse():
                     help="elements per launch (multiple of 16); 0 = the whole gradient in one launch. "
                          "The HBM-sizing workload is --elems 2800000000 --chunk 268435456")
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="CPU-baseline time budget; 0 skips it")
-    ap.add_argument("--legs", default="deq,acc,copy,cpu",
-                    help="extra legs after the timed quantize steps: deq, acc, copy, cpu, and (off by "
-                         "default) matrix, multi (comma list, '' = none)")
+    ap.add_argument("--legs", default="deq,acc,configs,wrapper,copy,cpu",
+                    help="extra legs after the timed quantize steps: deq, acc, configs, wrapper, copy, cpu, "
+                         "and (off by default) matrix, multi (comma list, '' = none)")
     return ap.parse_args()
 
 
@@ -90,7 +93,7 @@ def _time_passes(fn, budget_s, max_reps=10000):
             return reps, el
 
 
-def cpu_baseline(g_slab, r_slab, budget_s):
+def cpu_baseline(g_slab, r_slab, budget_s, thrd=THRD):
     """Time the CPU restatement of the reference kernel on a slab of the workload: the C version on
     all host threads (the headline baseline), on one thread, and the numpy version."""
     import numpy as np
@@ -99,12 +102,12 @@ def cpu_baseline(g_slab, r_slab, budget_s):
     n = g_slab.shape[0]
     c = np.empty((n + 15) // 16, dtype=np.uint32)
     r = r_slab.copy()
-    reps, el = _time_passes(lambda: oracle.c.fused_quantize_inplace(g_slab, r, c, THRD), budget_s * 0.6)
+    reps, el = _time_passes(lambda: oracle.c.fused_quantize_inplace(g_slab, r, c, thrd), budget_s * 0.6)
     oracle.c.set_threads(1)
-    reps1, el1 = _time_passes(lambda: oracle.c.fused_quantize_inplace(g_slab, r, c, THRD), budget_s * 0.2)
+    reps1, el1 = _time_passes(lambda: oracle.c.fused_quantize_inplace(g_slab, r, c, thrd), budget_s * 0.2)
     oracle.c.set_threads(threads)
     m = min(n, 1 << 22)
-    repsn, eln = _time_passes(lambda: oracle.vec.quantize(g_slab[:m], THRD, R_in=r_slab[:m]), budget_s * 0.2)
+    repsn, eln = _time_passes(lambda: oracle.vec.quantize(g_slab[:m], thrd, R_in=r_slab[:m]), budget_s * 0.2)
     return {
         "value": round(BYTES_QUANT * n * reps / el / 1e9, 3),
         "unit": "GB/s",
@@ -116,6 +119,242 @@ def cpu_baseline(g_slab, r_slab, budget_s):
         "one_thread_GBps": round(BYTES_QUANT * n * reps1 / el1 / 1e9, 3),
         "numpy_one_thread_GBps": round(BYTES_QUANT * m * repsn / eln / 1e9, 3),
     }
+
+
+def cpu_baseline_small(g, r0, thrd, budget_s, what):
+    """The same C restatement, all host threads, on another workload's own data."""
+    import numpy as np
+    import oracle
+    n = g.shape[0]
+    c = np.empty((n + 15) // 16, dtype=np.uint32)
+    r = r0.copy()
+    reps, el = _time_passes(lambda: oracle.c.fused_quantize_inplace(g, r, c, thrd), budget_s)
+    return {"value": round(BYTES_QUANT * n * reps / el / 1e9, 3), "unit": "GB/s", "cores": oracle.c.threads(),
+            "kind": "port", "elements_per_s": round(n * reps / el),
+            "sample": f"{reps} fused passes over {what} ({el:.1f} s)"}
+
+
+def source_stamp():
+    """First 16 hex digits of the SHA-256 of the kernel source: ties a counter summary under
+    profiles/ to the code it measured."""
+    import hashlib
+    with open(os.path.join(ROOT, "necklace_amd", "csrc", "nklq.hip"), "rb") as f:
+        return hashlib.sha256(f.read()).hexdigest()[:16]
+
+
+def hbm_traffic_from_profile(name):
+    """(bytes per launch, stale) from the committed rocprofv3 FETCH_SIZE / WRITE_SIZE summary: the
+    figure is only quoted when the summary was taken from the kernel source as it is now."""
+    import re
+    tpath = os.path.join(ROOT, "profiles", name)
+    if not os.path.exists(tpath):
+        return None, False
+    text = open(tpath).read()
+    m = re.search(r"^\s*total\s+([0-9,]+) B\s+vs algorithmic", text, re.M)
+    st = re.search(r"kernel source sha256\[:16\]:\s*([0-9a-f]{16})", text)
+    if not m:
+        return None, False
+    if not st or st.group(1) != source_stamp():
+        return None, True
+    return int(m.group(1).replace(",", "")), False
+
+
+def sparse_payloads(torch, k, words, gen, p_zero=0.9):
+    """[k, words] packed payloads (int32 bits) of i.i.d. codes: P(0) = p_zero, P(01) = P(10), never 11."""
+    half = (1.0 - p_zero) / 2
+    out = torch.empty(k, words, dtype=torch.int32, device="cuda")
+    shifts = (2 * torch.arange(16, device="cuda", dtype=torch.int64)).view(1, 16)
+    for p in range(k):
+        u = torch.rand(words, 16, device="cuda", generator=gen)
+        codes = (u < half).to(torch.int64) + 2 * ((u >= half) & (u < 2 * half)).to(torch.int64)
+        w = (codes << shifts).sum(-1)
+        out[p] = torch.where(w >= 2 ** 31, w - 2 ** 32, w).to(torch.int32)
+    return out
+
+
+def frac(gbps):
+    return round(gbps / HBM_PEAK_GBPS, 4)
+
+
+def bench_configs(torch, L, _lib, stream, gen, res, cpu_seconds):
+    """The four synthetic workloads that are not the headline one (BASELINE.json configs 1, 2, 3, 5)."""
+    import ctypes as ct
+    import numpy as np
+    check = _lib.check
+
+    # ---- config 1: 1,048,576 elements, N(0, 0.01), zero residual, thrd 0.005; flat and as 1024 x 1024
+    n1, t1 = 1 << 20, 0.005
+    g1 = torch.randn(n1, device="cuda", generator=gen) * 0.01
+    r1 = torch.zeros(n1, device="cuda")
+    c1 = torch.empty(n1 // 16, dtype=torch.int32, device="cuda")
+    f_flat = lambda: check(L.nklq_quantize_f32(g1.data_ptr(), r1.data_ptr(), r1.data_ptr(), c1.data_ptr(), n1, 1, t1, 1, stream))
+    f_sq = lambda: check(L.nklq_quantize_f32(g1.data_ptr(), r1.data_ptr(), r1.data_ptr(), c1.data_ptr(), 1024, 1024, t1, 1, stream))
+    out = {}
+    for name, f in (("flat", f_flat), ("square_1024x1024", f_sq)):
+        for _ in range(20):
+            f()
+        _, ev = time_region(torch, f, 500)
+        us = ev / 500 * 1e3
+        out[name] = {"us": round(us, 2), "GBps": round(BYTES_QUANT * n1 / us / 1e3, 1),
+                     "frac_hbm_peak": frac(BYTES_QUANT * n1 / us / 1e3), "elements_per_s": round(n1 / us * 1e6)}
+    out["note"] = "12.8 MB per launch: launch latency, not HBM, bounds it"
+    if cpu_seconds > 0:
+        out["cpu_baseline"] = cpu_baseline_small(g1.cpu().numpy(), np.zeros(n1, np.float32), t1, cpu_seconds * 0.1,
+                                                 "config 1's 1,048,576 elements")
+    res["config1"] = out
+
+    # ---- config 2: 25,557,032 elements = 161 segments, per-segment sigma log-uniform [1e-4, 1e-2], thrd 1e-3,
+    # 10 error-feedback steps with a fresh gradient each, packed as ONE flat vector (last word: 8 codes)
+    sizes = resnet50_sizes()
+    n2, t2, steps2 = sum(sizes), 1e-3, 10
+    sig = 10.0 ** (torch.rand(len(sizes), device="cuda", generator=gen) * 2 - 4)
+    scale = torch.repeat_interleave(sig, torch.tensor(sizes, device="cuda"))
+    grads = [torch.randn(n2, device="cuda", generator=gen) * scale for _ in range(steps2)]
+    r2 = torch.zeros(n2, device="cuda")
+    c2 = torch.empty(_lib.packed_words(n2), dtype=torch.int32, device="cuda")
+    state = {"i": 0}
+
+    def step2():
+        g = grads[state["i"] % steps2]
+        state["i"] += 1
+        check(L.nklq_quantize_f32(g.data_ptr(), r2.data_ptr(), r2.data_ptr(), c2.data_ptr(), n2, 1, t2, 1, stream))
+
+    for _ in range(steps2):
+        step2()
+    r2.zero_()
+    state["i"] = 0
+    _, ev = time_region(torch, step2, steps2)
+    us = ev / steps2 * 1e3
+    res["config2"] = {"elements": n2, "segments": len(sizes), "steps": steps2, "us_per_step": round(us, 2),
+                      "GBps": round(BYTES_QUANT * n2 / us / 1e3, 1), "frac_hbm_peak": frac(BYTES_QUANT * n2 / us / 1e3),
+                      "elements_per_s": round(n2 / us * 1e6),
+                      "note": "one launch per step over the flat vector; 10 different gradients (1 GB) so "
+                              "that no step finds its input in the 256 MB memory-side cache"}
+    if cpu_seconds > 0:
+        res["config2"]["cpu_baseline"] = cpu_baseline_small(grads[0].cpu().numpy(), np.zeros(n2, np.float32), t2,
+                                                            cpu_seconds * 0.2, "config 2's 25,557,032 elements")
+    del grads, scale, r2, c2
+
+    # ---- config 3: 64 buckets of 1M..8M elements (not multiples of 16), 8 payloads each (local + 7 peers,
+    # P(0) = 0.9), fixed-order sum into a fresh fp32 buffer
+    rng = np.random.default_rng(3)
+    lens = []
+    while len(lens) < 64:
+        v = int(rng.integers(1_000_000, 8_000_001))
+        if v % 16:
+            lens.append(v)
+    words = [_lib.packed_words(v) for v in lens]
+    woff = np.concatenate([[0], np.cumsum([-(-w // 16) * 16 for w in words])]).astype(np.int64)  # 64 B aligned
+    total_words, total = int(woff[-1]), sum(lens)
+    msgs = sparse_payloads(torch, K_PAYLOADS, total_words, gen)      # one contiguous message per worker
+    accs = [torch.empty(v, device="cuda") for v in lens]
+    ptr_tabs = [(ct.c_void_p * K_PAYLOADS)(*[msgs[p].data_ptr() + 4 * int(woff[b]) for p in range(K_PAYLOADS)])
+                for b in range(64)]
+
+    def per_bucket():
+        for b in range(64):
+            check(L.nklq_dequant_accumulate_f32(accs[b].data_ptr(), ptr_tabs[b], K_PAYLOADS, lens[b], 1e-3, 0, stream))
+
+    acc_arr = (ct.c_void_p * 64)(*[a.data_ptr() for a in accs])
+    n_arr = (ct.c_uint64 * 64)(*lens)
+    wo_arr = (ct.c_uint64 * 64)(*[int(w) for w in woff[:64]])
+    base_arr = (ct.c_void_p * K_PAYLOADS)(*[msgs[p].data_ptr() for p in range(K_PAYLOADS)])
+
+    def one_launch():
+        check(L.nklq_dequant_accumulate_multi_f32(64, acc_arr, n_arr, wo_arr, base_arr, K_PAYLOADS, 1e-3, 0, 1.0, stream))
+
+    c3 = {"buckets": 64, "payloads": K_PAYLOADS, "elements": total}
+    byt = (0.25 * K_PAYLOADS + 4) * total
+    for name, f in (("one_launch_per_bucket", per_bucket), ("all_buckets_one_launch", one_launch)):
+        for _ in range(3):
+            f()
+        _, ev = time_region(torch, f, 10)
+        ms = ev / 10
+        c3[name] = {"ms": round(ms, 4), "elements_per_s": round(total / ms * 1e3), "GBps": round(byt / ms / 1e6, 1),
+                    "frac_hbm_peak": frac(byt / ms / 1e6)}
+    res["config3"] = c3
+    del msgs, accs
+
+    # ---- config 5: 2.8e9 elements (11.2 GB + 11.2 GB + 0.7 GB resident), N(0, 5e-3), thrd 1e-2, 5 steps in
+    # chunks of 268,435,456 elements
+    n5, t5, chunk5, steps5 = 2_800_000_000, 1e-2, 268_435_456, 5
+    free, _ = torch.cuda.mem_get_info()
+    if free > 2 * 4 * n5 + n5 // 4 + (4 << 30):
+        g5 = torch.empty(n5, device="cuda")
+        for lo in range(0, n5, 1 << 28):
+            hi = min(n5, lo + (1 << 28))
+            torch.randn(hi - lo, device="cuda", generator=gen, out=g5[lo:hi])
+            g5[lo:hi] *= 5e-3
+        r5 = torch.zeros(n5, device="cuda")
+        c5 = torch.empty(_lib.packed_words(n5), dtype=torch.int32, device="cuda")
+        pieces = [(lo, min(n5, lo + chunk5)) for lo in range(0, n5, chunk5)]
+        gp, rp, cp = g5.data_ptr(), r5.data_ptr(), c5.data_ptr()
+
+        def step5():
+            for lo, hi in pieces:
+                check(L.nklq_quantize_f32(gp + 4 * lo, rp + 4 * lo, rp + 4 * lo, cp + 4 * (lo // 16), hi - lo, 1, t5, 1, stream))
+
+        step5()
+        r5.zero_()
+        _, ev = time_region(torch, step5, steps5)
+        ms = ev / steps5
+        res["config5"] = {"elements": n5, "chunk": chunk5, "launches_per_step": len(pieces), "steps": steps5,
+                          "ms_per_step": round(ms, 4), "GBps": round(BYTES_QUANT * n5 / ms / 1e6, 1),
+                          "frac_hbm_peak": frac(BYTES_QUANT * n5 / ms / 1e6), "elements_per_s": round(n5 / ms * 1e3),
+                          "resident_GB": round((2 * 4 * n5 + 4 * _lib.packed_words(n5)) / 1e9, 2)}
+        del g5, r5, c5
+    else:
+        res["config5"] = {"skipped": f"only {free / 1e9:.0f} GB of HBM free"}
+
+
+def bench_wrapper(torch, L, _lib, stream, res):
+    """Wall time per call of the reference-named wrapper (necklace/cuda/quantize.py:96-115 creates a
+    stream and blocks on it every call) at sizes where the kernel takes a few microseconds."""
+    from necklace_amd.cuda import quantize as q
+    out = {}
+    for name, shape in (("1048576", (1 << 20,)), ("224x224", (224, 224))):
+        A = torch.randn(*shape, device="cuda") * 0.01
+        R = torch.zeros_like(A)
+        m = (shape[0] + 15) // 16
+        C = torch.empty((m,) + tuple(shape[1:]), dtype=torch.int32, device="cuda")
+        n, k = (shape[0], 1) if len(shape) == 1 else shape
+        raw = lambda: _lib.check(L.nklq_quantize_f32(A.data_ptr(), R.data_ptr(), R.data_ptr(), C.data_ptr(), n, k, 0.005, 1, stream))
+        for _ in range(50):
+            raw()
+        _, ev = time_region(torch, raw, 1000)
+        row = {"kernel_us": round(ev, 2)}          # ev is ms for 1000 launches = us per launch
+        for label, kw in (("sync_true", {}), ("sync_false", {"sync": False})):
+            f = lambda: q.cu_fn_matrix_quantize_e(A, C, R, 0.005, add_residual=True, **kw)
+            for _ in range(50):
+                f()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(1000):
+                f()
+            torch.cuda.synchronize()
+            row[f"wall_us_per_call_{label}"] = round((time.perf_counter() - t0) * 1e3, 2)
+        t0 = time.perf_counter()
+        for _ in range(1000):
+            raw()
+        torch.cuda.synchronize()
+        row["wall_us_per_call_c_abi_async"] = round((time.perf_counter() - t0) * 1e3, 2)
+        out[name] = row
+    res["wrapper_call_overhead"] = out
+
+
+def resnet50_sizes():
+    """Element counts of ResNet-50's 161 parameter tensors, in module order (25,557,032 in all)."""
+    sizes = [64 * 3 * 7 * 7, 64, 64]
+    inpl = 64
+    for planes, blocks in ((64, 3), (128, 4), (256, 6), (512, 3)):
+        for b in range(blocks):
+            sizes += [planes * inpl, planes, planes, planes * planes * 9, planes, planes,
+                      4 * planes * planes, 4 * planes, 4 * planes]
+            if b == 0:
+                sizes += [4 * planes * inpl, 4 * planes, 4 * planes]
+            inpl = 4 * planes
+    sizes += [1000 * 2048, 1000]
+    return sizes
 
 
 def main():
@@ -176,14 +415,12 @@ def main():
     singles = sorted(e0.elapsed_time(e1) for e0, e1 in pairs)
 
     # HBM bytes per launch from the rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this same command
-    # (a separate, committed measurement: counters cannot be read from inside the process)
-    traffic = None
-    tpath = os.path.join(ROOT, "profiles", "quant_flat_355M_pmc.txt")
-    if os.path.exists(tpath) and n == N_ELEMS and len(pieces) == 1:
-        import re
-        m = re.search(r"^\s*total\s+([0-9,]+) B\s+vs algorithmic", open(tpath).read(), re.M)
-        if m:
-            traffic = int(m.group(1).replace(",", ""))
+    # (a separate, committed measurement: counters cannot be read from inside the process).  The
+    # summary carries the hash of the kernel source it was taken from; after any change to the
+    # source the figure is withheld until the counters have been collected again.
+    traffic, traffic_stale = None, False
+    if n == N_ELEMS and len(pieces) == 1:
+        traffic, traffic_stale = hbm_traffic_from_profile("quant_flat_355M_pmc.txt")
 
     res = {
         "metric": "fused 2-bit quantize GB/s (355M fp32 grad)" if n == N_ELEMS
@@ -221,7 +458,9 @@ def main():
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
             "traffic": traffic,
+            "traffic_stale": traffic_stale,
             "kernel": "quant_flat_kernel",
+            "kernel_source_sha256_16": source_stamp(),
             "bytes_per_launch": bytes_per_launch,
             "avg_launch_ms": round(kernel_ms, 4),
         },
@@ -276,6 +515,8 @@ def main():
             "elements_per_s": round(nb / (acc_ms * 1e-3)),
             "ms": round(acc_ms, 4),
             "GBps": round(acc_bytes / (acc_ms * 1e-3) / 1e9, 1),
+            "frac_hbm_peak": frac(acc_bytes / (acc_ms * 1e-3) / 1e9),
+            "note": "50 MB working set: served by the 256 MB memory-side cache when repeated",
         }
         del payloads, acc
         # the same sum at gradient size: 8 random payloads (the kernel's time does not depend on the codes)
@@ -289,7 +530,7 @@ def main():
             def accum_large():
                 _lib.check(L.nklq_dequant_accumulate_f32(accl.data_ptr(), ptrl, K_PAYLOADS, n, THRD, 0, stream))
 
-            for _ in range(3):
+            for _ in range(25):  # the first few dozen launches on fresh buffers run 2-5 % slower
                 accum_large()
             _, ev = time_region(torch, accum_large, 20)
             res["dequant_accumulate_large"] = {
@@ -297,8 +538,15 @@ def main():
                 "elements_per_s": round(n / (ev / 20 * 1e-3)),
                 "ms": round(ev / 20, 4),
                 "GBps": round((0.25 * K_PAYLOADS + 4) * n / (ev / 20 * 1e-3) / 1e9, 1),
+                "frac_hbm_peak": frac((0.25 * K_PAYLOADS + 4) * n / (ev / 20 * 1e-3) / 1e9),
             }
             del big, accl
+
+    if "configs" in legs and n == N_ELEMS:
+        bench_configs(torch, L, _lib, stream, gen, res, args.cpu_seconds if "cpu" in legs else 0.0)
+
+    if "wrapper" in legs:
+        bench_wrapper(torch, L, _lib, stream, res)
 
     if "matrix" in legs:
         # the reference's own layout: (n, k) matrix, codes packed down the columns

@@ -92,6 +92,35 @@ def _finish(stream, device, sync):
         stream.synchronize()
 
 
+class _on_device:
+    """`with torch.cuda.device(d)` only when d is not already the current device: the library launches
+    on the current HIP device, and switching back and forth costs more than a small kernel takes."""
+    __slots__ = ("ctx",)
+
+    def __init__(self, device):
+        self.ctx = None if device.index == torch.cuda.current_device() else torch.cuda.device(device)
+
+    def __enter__(self):
+        if self.ctx is not None:
+            self.ctx.__enter__()
+
+    def __exit__(self, *exc):
+        if self.ctx is not None:
+            return self.ctx.__exit__(*exc)
+        return False
+
+
+_fn_cache = {}
+
+
+def _fn(name):
+    """The bound ctypes function, looked up once."""
+    f = _fn_cache.get(name)
+    if f is None:
+        f = _fn_cache[name] = getattr(_lib.lib(), name)
+    return f
+
+
 def _quantize(A, C, R, thrd, add_residual, stream, sync):
     _check_f32("A", A)
     _check_f32("R", R)
@@ -99,26 +128,32 @@ def _quantize(A, C, R, thrd, add_residual, stream, sync):
         raise ValueError(f"A {tuple(A.shape)} and R {tuple(R.shape)} differ in shape")
     n, k = _shape2(A)
     _check_words("C", C, n, k, A.dim())
-    if not (A.device == R.device == C.device):
+    dev = A.device
+    if not (dev == R.device == C.device):
         raise ValueError("A, C and R must be on the same GPU")
-    with torch.cuda.device(A.device):
-        h = nbutils.stream_handle(stream, A.device)
-        _lib.check(_lib.lib().nklq_quantize_f32(
-            A.data_ptr(), R.data_ptr() if add_residual else None, R.data_ptr(), C.data_ptr(),
-            n, k, float(thrd), 1 if add_residual else 0, h))
-        _finish(stream, A.device, sync)
+    with _on_device(dev):
+        h = nbutils.stream_handle(stream, dev)
+        rp = R.data_ptr()
+        code = _fn("nklq_quantize_f32")(A.data_ptr(), rp if add_residual else None, rp, C.data_ptr(),
+                                        n, k, float(thrd), 1 if add_residual else 0, h)
+        if code:
+            _lib.check(code)
+        _finish(stream, dev, sync)
 
 
 def _dequantize(A, C, thrd, stream, sync):
     _check_f32("A", A)
     n, k = _shape2(A)
     _check_words("C", C, n, k, A.dim())
-    if A.device != C.device:
+    dev = A.device
+    if dev != C.device:
         raise ValueError("A and C must be on the same GPU")
-    with torch.cuda.device(A.device):
-        h = nbutils.stream_handle(stream, A.device)
-        _lib.check(_lib.lib().nklq_dequantize_f32(A.data_ptr(), C.data_ptr(), n, k, float(thrd), h))
-        _finish(stream, A.device, sync)
+    with _on_device(dev):
+        h = nbutils.stream_handle(stream, dev)
+        code = _fn("nklq_dequantize_f32")(A.data_ptr(), C.data_ptr(), n, k, float(thrd), h)
+        if code:
+            _lib.check(code)
+        _finish(stream, dev, sync)
 
 
 class _Kernel:
@@ -207,7 +242,7 @@ def cu_fn_dequantize_accumulate_e(acc, payloads, thrd=0.3, accumulate=False, str
         if p.device != acc.device:
             raise ValueError("acc and payloads must be on the same GPU")
     ptrs = (ct.c_void_p * len(payloads))(*[p.data_ptr() for p in payloads])
-    with torch.cuda.device(acc.device):
+    with _on_device(acc.device):
         h = nbutils.stream_handle(stream, acc.device)
         _lib.check(_lib.lib().nklq_dequant_accumulate_f32(
             acc.data_ptr(), ptrs, len(payloads), n, float(thrd), 1 if accumulate else 0, h))
@@ -245,7 +280,7 @@ def cu_fn_quantize_multi_e(grads, comps, resis, thrd=0.3, add_residual=True, str
         if not (gr.device == cm.device == rs.device == dev):
             raise ValueError("all tensors must be on the same GPU")
         ns.append(n)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         h = nbutils.stream_handle(stream, dev)
         _lib.check(_lib.lib().nklq_quantize_multi_f32(
             len(ns), _ptr_array([t.data_ptr() for t in grads]), _ptr_array([t.data_ptr() for t in resis]),
@@ -289,7 +324,7 @@ def cu_fn_dequantize_accumulate_multi_e(accs, word_offsets, payloads, thrd=0.3, 
         if wo < 0 or wo + packed_rows(n) > w_total:
             raise ValueError(f"vector {i}: words [{wo}, {wo + packed_rows(n)}) exceed the payload length {w_total}")
         ns.append(n)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         h = nbutils.stream_handle(stream, dev)
         _lib.check(_lib.lib().nklq_dequant_accumulate_multi_f32(
             len(ns), _ptr_array([t.data_ptr() for t in accs]), (ct.c_uint64 * len(ns))(*ns),

@@ -166,7 +166,7 @@ class GradCompressor:
         m, g_arr, r_arr, c_arr, n_arr, _ = self._tables(grads, "gradient")
         if not m:
             return
-        with torch.cuda.device(self.resi.device):
+        with _q._on_device(self.resi.device):
             _lib.check(_lib.lib().nklq_quantize_multi_f32(
                 m, g_arr, r_arr, c_arr, n_arr, self.thrd, 1, _nb.stream_handle(stream, self.resi.device)))
         if sync:
@@ -196,7 +196,7 @@ class GradCompressor:
         m, o_arr, _, _, n_arr, wo_arr = self._tables(outs, "output")
         if not m:
             return
-        with torch.cuda.device(self.resi.device):
+        with _q._on_device(self.resi.device):
             _lib.check(_lib.lib().nklq_dequant_accumulate_multi_f32(
                 m, o_arr, n_arr, wo_arr, self._pl_arr, self.kn, self.thrd, 0,
                 float(self.kn) if average else 1.0, _nb.stream_handle(stream, self.resi.device)))
