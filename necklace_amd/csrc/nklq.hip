@@ -137,29 +137,6 @@ __device__ __forceinline__ void st4(float* p, f32x4 v)
     }
 }
 
-// Store of a lane's 16 bytes inside a wave's 1 KiB piece that may start anywhere: the first and
-// the last 128-byte line of a piece that starts off a line are shared with the neighbouring pieces
-// (other waves).  A streaming (non-temporal) store of part of a line goes to memory as a
-// partial-line write; that is harmless when the cut falls on a 32-byte sector, but a cut inside a
-// sector makes memory read, merge and write the sector.  In that case the lanes on those two lines
-// store with the ordinary policy instead, so that the halves meet in L2 (the neighbouring piece is
-// written from the same XCD, and the line is already there from the residual's load) and leave it
-// as whole sectors.
-template <bool ALIGNED, bool NT>
-__device__ __forceinline__ void st4_piece(float* p, f32x4 v, int lane)
-{
-    if constexpr (NT) {
-        const uintptr_t a = reinterpret_cast<uintptr_t>(p);
-        const uintptr_t piece = a - (uintptr_t)lane * 16;  // lane 0's address
-        const bool cut_in_sector = (piece & 31u) != 0;
-        const bool edge = cut_in_sector && ((a >> 7) == (piece >> 7) || ((a + 15) >> 7) == ((piece + 1023) >> 7));
-        if (edge) st4<ALIGNED, false>(p, v);
-        else st4<ALIGNED, true>(p, v);
-    } else {
-        st4<ALIGNED, false>(p, v);
-    }
-}
-
 // ---------------------------------------------------------------- chunk -> workgroup map
 
 // Workgroups are handed to the XCDs round-robin by workgroup id.  With
@@ -251,6 +228,45 @@ __global__ __launch_bounds__(BLOCK) void quant_flat_kernel(
     }
 }
 
+// The same pass for a residual that does not start on a 128-byte line (a view cut out of a larger
+// buffer at any element): every chunk's first and last line is then shared with the neighbouring
+// chunk, and written from two XCDs the two parts reach memory as two partial-line writes.  Here
+// chunks are dealt to the XCDs in runs of 16 (workgroup b runs on XCD b % 8; a run of 16 chunks = 4
+// consecutive workgroups of ONE XCD, the next run goes to the next XCD), so that all but one
+// boundary in 16 lies inside one XCD's L2, where the parts merge.  One chunk per wave, 256-thread
+// workgroups.
+constexpr uint32_t kRunChunks = 16;
+
+template <bool ALIGNED, bool ADD, bool NT>
+__global__ __launch_bounds__(256) void quant_flat_offline_kernel(
+    const float* g, const float* rin, float* rout, uint32_t* __restrict__ c, uint64_t n,
+    uint64_t n_chunks, uint32_t has_tail, float t)
+{
+    if (has_tail && blockIdx.x == gridDim.x - 1) {
+        quant_tail<ADD, 256>(g, rin, rout, c, n_chunks * kChunk, n, t);
+        return;
+    }
+    const int lane = threadIdx.x & (kWave - 1);
+    const uint32_t w = threadIdx.x >> 6;
+    const uint32_t xcd = blockIdx.x & 7u;
+    const uint32_t j = blockIdx.x >> 3;
+    const uint64_t run = (uint64_t)(j >> 2) * 8 + xcd;
+    const uint64_t ch = run * kRunChunks + (j & 3u) * 4 + w;
+    if (ch >= n_chunks) return;
+    f32x4 v = ld4<ALIGNED, NT>(g + ch * kChunk + lane * 4);
+    if constexpr (ADD) v = v + ld4<ALIGNED, NT>(rin + ch * kChunk + lane * 4);
+    float o0, o1, o2, o3;
+    uint32_t b = quant_one(v.x, t, o0);
+    b |= quant_one(v.y, t, o1) << 2;
+    b |= quant_one(v.z, t, o2) << 4;
+    b |= quant_one(v.w, t, o3) << 6;
+    f32x4 o;
+    o.x = o0; o.y = o1; o.z = o2; o.w = o3;
+    st4<ALIGNED, NT>(rout + ch * kChunk + lane * 4, o);
+    const uint32_t word = quad_or(b << (8 * (lane & 3)));
+    if ((lane & 3) == 0) c[ch * kWordsPerChunk + (lane >> 2)] = word;
+}
+
 // ---------------------------------------------------------------- flat dequantize
 
 // out[j] = decode(c)[j]  (the reference dequantize, flat).  The 4 lanes of a quad read the
@@ -280,6 +296,35 @@ __global__ __launch_bounds__(BLOCK) void deq_flat_kernel(
         if (ch >= n_chunks) continue;
         const uint32_t word = c[ch * kWordsPerChunk + (lane >> 2)];
         st4<ALIGNED, NT>(out + ch * kChunk + lane * 4, deq_byte((word >> sh) & 0xFFu, t));
+    }
+}
+
+// Decode into a vector that does not start on a 128-byte line: the chunk grid is moved left by the
+// d = 0..31 elements the vector's start lies past a line, so that every wave still writes whole,
+// aligned lines: chunk j covers elements [256 j - d, 256 j - d + 256), clipped to the vector.  A
+// lane's 4 elements then start at any code position, possibly across two words: the 8 bits are
+// cut out of the 64-bit pair.  Only the first and the last quad can be partial (element by element).
+template <bool NT>
+__global__ __launch_bounds__(256) void deq_flat_shift_kernel(float* out, const uint32_t* __restrict__ c,
+                                                             uint64_t n, uint64_t n_chunks, uint32_t d, float t)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    const uint64_t ch = (uint64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (ch >= n_chunks) return;
+    const int64_t e = (int64_t)(ch * kChunk) - (int64_t)d + lane * 4;
+    if (e >= (int64_t)n || e + 4 <= 0) return;
+    if (e >= 0 && e + 4 <= (int64_t)n) {
+        const uint64_t wi = (uint64_t)e >> 4;
+        const uint32_t sh = 2 * (uint32_t)(e & 15);
+        uint64_t bits = c[wi];
+        if (sh > 24) bits |= (uint64_t)c[wi + 1] << 32;  // the quad reaches into the next word (e + 3 < n: it exists)
+        st4<true, NT>(out + e, deq_byte((uint32_t)(bits >> sh) & 0xFFu, t));
+    } else {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int64_t ek = e + k;
+            if (ek >= 0 && ek < (int64_t)n) out[ek] = deq_code((c[ek >> 4] >> (2 * (uint32_t)(ek & 15))) & 3u, t);
+        }
     }
 }
 
@@ -479,8 +524,13 @@ constexpr int kRowsBlock = 16 * kWave;  // 1024 threads
 // two halves merge in that XCD's L2 into a full-line write, written from two XCDs they reach memory
 // as two partial-line writes.  Returns false for the padding workgroups of the last group of rows.
 __device__ __forceinline__ bool rows_tile_of(uint32_t b, uint32_t col_tiles, uint64_t m, uint64_t* x,
-                                             uint32_t* T)
+                                             uint32_t* T, uint32_t pinned = 1)
 {
+    if (!pinned) {
+        *x = b / col_tiles;
+        *T = b % col_tiles;
+        return *x < m;
+    }
     const uint32_t e = b & 7u;
     const uint32_t j = b >> 3;
     *x = (uint64_t)(j / col_tiles) * 8 + e;
@@ -488,71 +538,86 @@ __device__ __forceinline__ bool rows_tile_of(uint32_t b, uint32_t col_tiles, uin
     return *x < m;
 }
 
+// (Two or four 1 KiB pieces per wave and array, i.e. tiles of 512 or 1024 columns, measured 3-12 %
+// slower than one.)
 template <bool ADD, bool NT, bool ALIGNED>
 __global__ __launch_bounds__(kRowsBlock) void quant_2d_rows_kernel(
     const float* g, const float* rin, float* rout, uint32_t* __restrict__ c, uint64_t n,
-    uint64_t k, uint32_t col_tiles, float t)
+    uint64_t k, uint32_t col_tiles, float t, uint32_t pinned)
 {
-    __shared__ uint32_t words[256];
+    constexpr int CQ = 1;        // 1 KiB pieces per wave and array
+    constexpr int W = 256 * CQ;  // columns per tile
+    __shared__ uint32_t words[W];
     const int lane = threadIdx.x & (kWave - 1);
     const uint32_t i = threadIdx.x >> 6;  // row inside the tile = code position inside the word
     uint64_t x;
     uint32_t T;
-    if (!rows_tile_of(blockIdx.x, col_tiles, (n + 15) / 16, &x, &T)) return;
-    const uint64_t y0 = (uint64_t)T * 256;
-    const uint64_t y = y0 + (uint64_t)lane * 4;
+    if (!rows_tile_of(blockIdx.x, col_tiles, (n + 15) / 16, &x, &T, pinned)) return;
+    const uint64_t y0 = (uint64_t)T * W;
     const uint64_t row = x * 16 + i;
-    // columns this lane owns: 4, or fewer at the right edge, or none
-    // (with ALIGNED, k is a multiple of 4: it is 4 or none)
-    const int cnt = (row < n && y < k) ? ((ALIGNED || k - y >= 4) ? 4 : (int)(k - y)) : 0;
-    const uint64_t off = row * k + y;
-    float a[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-    float r[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-    if (cnt == 4) {
-        const f32x4 va = ld4<ALIGNED, NT>(g + off);
-        a[0] = va.x; a[1] = va.y; a[2] = va.z; a[3] = va.w;
-        if constexpr (ADD) {
-            const f32x4 vr = ld4<ALIGNED, NT>(rin + off);
-            r[0] = vr.x; r[1] = vr.y; r[2] = vr.z; r[3] = vr.w;
-        }
-    } else {
+    int cnt[CQ];
+    uint64_t off[CQ];
+    float a[CQ][4], r[CQ][4];
 #pragma unroll
-        for (int j = 0; j < 3; ++j) {
-            if (j < cnt) {
-                a[j] = g[off + j];
-                if constexpr (ADD) r[j] = rin[off + j];
+    for (int q = 0; q < CQ; ++q) {
+        const uint64_t y = y0 + 256 * q + (uint64_t)lane * 4;
+        // columns this lane owns in piece q: 4, or fewer at the right edge, or none
+        // (with ALIGNED, k is a multiple of 4: it is 4 or none)
+        cnt[q] = (row < n && y < k) ? ((ALIGNED || k - y >= 4) ? 4 : (int)(k - y)) : 0;
+        off[q] = row * k + y;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { a[q][j] = 0.0f; r[q][j] = 0.0f; }
+        if (cnt[q] == 4) {
+            const f32x4 va = ld4<ALIGNED, NT>(g + off[q]);
+            a[q][0] = va.x; a[q][1] = va.y; a[q][2] = va.z; a[q][3] = va.w;
+            if constexpr (ADD) {
+                const f32x4 vr = ld4<ALIGNED, NT>(rin + off[q]);
+                r[q][0] = vr.x; r[q][1] = vr.y; r[q][2] = vr.z; r[q][3] = vr.w;
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 3; ++j) {
+                if (j < cnt[q]) {
+                    a[q][j] = g[off[q] + j];
+                    if constexpr (ADD) r[q][j] = rin[off[q] + j];
+                }
             }
         }
     }
-    if (threadIdx.x < 256) words[threadIdx.x] = 0;
+    for (int wi = threadIdx.x; wi < W; wi += kRowsBlock) words[wi] = 0;
     __syncthreads();
-    if (cnt > 0) {
-        float o[4];
-        uint32_t code[4];
+    const uint32_t sh = 2 * i;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            float v = a[j];
-            if constexpr (ADD) v = v + r[j];
-            code[j] = quant_one(v, t, o[j]);
+    for (int q = 0; q < CQ; ++q) {
+        if (cnt[q] > 0) {
+            float o[4];
+            uint32_t code[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                float v = a[q][j];
+                if constexpr (ADD) v = v + r[q][j];
+                code[j] = quant_one(v, t, o[j]);
+            }
+            if (cnt[q] == 4) {
+                f32x4 vo;
+                vo.x = o[0]; vo.y = o[1]; vo.z = o[2]; vo.w = o[3];
+                st4<ALIGNED, NT>(rout + off[q], vo);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 3; ++j)
+                    if (j < cnt[q]) rout[off[q] + j] = o[j];
+            }
+            // column 256 q + 4 lane + j lives at words[256 q + 64 j + lane]: consecutive lanes, consecutive banks
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (j < cnt[q] && code[j]) atomicOr(&words[256 * q + 64 * j + lane], code[j] << sh);
         }
-        if (cnt == 4) {
-            f32x4 vo;
-            vo.x = o[0]; vo.y = o[1]; vo.z = o[2]; vo.w = o[3];
-            st4_piece<ALIGNED, NT>(rout + off, vo, lane);
-        } else {
-#pragma unroll
-            for (int j = 0; j < 3; ++j)
-                if (j < cnt) rout[off + j] = o[j];
-        }
-        const uint32_t sh = 2 * i;
-        // column 4*lane + j lives at words[64*j + lane]: consecutive lanes, consecutive banks
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-            if (j < cnt && code[j]) atomicOr(&words[64 * j + lane], code[j] << sh);
     }
     __syncthreads();
-    if (threadIdx.x < 256 && y0 + threadIdx.x < k)
-        c[x * k + y0 + threadIdx.x] = words[64 * (threadIdx.x & 3) + (threadIdx.x >> 2)];
+    for (int wi = threadIdx.x; wi < W; wi += kRowsBlock) {
+        const int q = wi >> 8, cq = wi & 255;
+        if (y0 + wi < k) c[x * k + y0 + wi] = words[256 * q + 64 * (cq & 3) + (cq >> 2)];
+    }
 }
 
 // Decode of a tile.  SHIFT = false: every row starts on a 128-byte line (k a multiple of 32, base
@@ -1119,9 +1184,38 @@ int launch_acc_flat(float* acc, const PayloadPtrs& pl, int k, uint64_t n, float 
         default: return NKLQ_ERANGE;                             \
     }
 
+// Residual views that do not start on a 128-byte line take the kernel that keeps shared lines whole.
+int launch_quant_flat_offline(const float* g, const float* rin, float* rout, uint32_t* c, uint64_t n, float t,
+                              bool add, bool al, hipStream_t s)
+{
+    const uint64_t n_chunks = n / kChunk;
+    const uint32_t has_tail = (n_chunks * kChunk < n) ? 1u : 0u;
+    const uint64_t runs8 = ((n_chunks + kRunChunks - 1) / kRunChunks + 7) / 8 * 8;  // runs, in groups of 8 XCDs
+    const uint64_t work = runs8 * (kRunChunks / 4);
+    if (work + has_tail > 0x7FFFFFFFull) return NKLQ_ERANGE;
+    const dim3 grid((uint32_t)work + has_tail), block(256);
+    const bool nt = tk.nontemporal != 0;
+#define NKLQ_QO(AL, ADD, NT) \
+    launch_kernel((quant_flat_offline_kernel<AL, ADD, NT>), grid, block, 0, s, g, rin, rout, c, n, n_chunks, has_tail, t)
+    switch ((al ? 4 : 0) | (add ? 2 : 0) | (nt ? 1 : 0)) {
+        case 7: NKLQ_QO(true, true, true); break;
+        case 6: NKLQ_QO(true, true, false); break;
+        case 5: NKLQ_QO(true, false, true); break;
+        case 4: NKLQ_QO(true, false, false); break;
+        case 3: NKLQ_QO(false, true, true); break;
+        case 2: NKLQ_QO(false, true, false); break;
+        case 1: NKLQ_QO(false, false, true); break;
+        default: NKLQ_QO(false, false, false); break;
+    }
+#undef NKLQ_QO
+    return launch_status();
+}
+
 int dispatch_quant_flat(const float* g, const float* rin, float* rout, uint32_t* c, uint64_t n,
                         float t, bool add, bool al, hipStream_t s)
 {
+    if ((reinterpret_cast<uintptr_t>(rout) & 127u) != 0 && n >= kChunk)
+        return launch_quant_flat_offline(g, rin, rout, c, n, t, add, al, s);
 #define NKLQ_CALL(U, B) launch_quant_flat<U, B>(g, rin, rout, c, n, t, add, al, s)
     NKLQ_FOR_GEOMETRY(NKLQ_CALL)
 #undef NKLQ_CALL
@@ -1129,6 +1223,17 @@ int dispatch_quant_flat(const float* g, const float* rin, float* rout, uint32_t*
 
 int dispatch_deq_flat(float* out, const uint32_t* c, uint64_t n, float t, hipStream_t s)
 {
+    const uint32_t d = (uint32_t)((reinterpret_cast<uintptr_t>(out) >> 2) & 31u);  // elements past a 128-byte line
+    if (d != 0) {
+        const uint64_t n_chunks = (n + d + kChunk - 1) / kChunk;
+        const uint64_t blocks = (n_chunks + 3) / 4;
+        if (blocks > 0x7FFFFFFFull) return NKLQ_ERANGE;
+        if (tk.nontemporal)
+            launch_kernel((deq_flat_shift_kernel<true>), dim3((uint32_t)blocks), dim3(256), 0, s, out, c, n, n_chunks, d, t);
+        else
+            launch_kernel((deq_flat_shift_kernel<false>), dim3((uint32_t)blocks), dim3(256), 0, s, out, c, n, n_chunks, d, t);
+        return launch_status();
+    }
 #define NKLQ_CALL(U, B) launch_deq_flat<U, B>(out, c, n, t, s)
     NKLQ_FOR_GEOMETRY(NKLQ_CALL)
 #undef NKLQ_CALL
@@ -1327,13 +1432,16 @@ int nklq_quantize_f32(const float* g, const float* r_in, float* r_out, uint32_t*
         return launch_status();
     }
     const bool al = (n_cols % 4 == 0) && aligned16(g) && aligned16(r_out) && (!add || aligned16(r_in));
+    // rows that do not all start on a 128-byte line: neighbouring tiles of a row share lines, keep them on one XCD
+    const bool on_lines = (n_cols % 32 == 0) && (reinterpret_cast<uintptr_t>(r_out) & 127u) == 0;
+    const uint32_t pinned = on_lines ? 0u : 1u;
     const uint64_t col_tiles = (n_cols + 255) / 256;
-    const uint64_t m8 = (m + 7) / 8 * 8;  // word rows are dealt to the XCDs in groups of 8
+    const uint64_t m8 = pinned ? (m + 7) / 8 * 8 : m;  // pinned: word rows are dealt to the XCDs in groups of 8
     if (col_tiles > 0x7FFFFFFFull || m8 > 0x7FFFFFFFull / col_tiles) return NKLQ_ERANGE;
     const dim3 grid((uint32_t)(m8 * col_tiles)), block(kRowsBlock);
-#define NKLQ_Q2(ADD, NT, AL)                                                                         \
+#define NKLQ_Q2(ADD, NT, AL)                                                                        \
     launch_kernel((quant_2d_rows_kernel<ADD, NT, AL>), grid, block, 0, s, g, r_in, r_out, c, n_rows, \
-                       n_cols, (uint32_t)col_tiles, thrd)
+                  n_cols, (uint32_t)col_tiles, thrd, pinned)
     switch ((add ? 4 : 0) | (tk.nontemporal ? 2 : 0) | (al ? 1 : 0)) {
         case 7: NKLQ_Q2(true, true, true); break;
         case 6: NKLQ_Q2(true, true, false); break;
