@@ -549,28 +549,35 @@ def main():
         bench_wrapper(torch, L, _lib, stream, res)
 
     if "matrix" in legs:
-        # the reference's own layout: (n, k) matrix, codes packed down the columns
-        side = 8192
-        A = g[:side * side].view(side, side)
-        R = torch.zeros(side, side, device="cuda")
-        C = torch.empty(side // 16, side, dtype=torch.int32, device="cuda")
+        # the reference's own layout: (n, k) matrix, codes packed down the columns; wide and narrow,
+        # rows on and off 128-byte lines
+        res["matrix"] = {}
+        for rows, cols in ((8192, 8192), (8191, 8191), (16384, 16383), (100000, 1000), (20_000_000, 3),
+                           (4_000_000, 17), (1_000_000, 65)):
+            tot = rows * cols
+            A = g[:tot] if tot <= n else torch.randn(tot, device="cuda", generator=gen) * 1e-3
+            R = torch.zeros(tot, device="cuda")
+            C = torch.empty(_lib.packed_words(rows, cols), dtype=torch.int32, device="cuda")
 
-        def mq():
-            _lib.check(L.nklq_quantize_f32(A.data_ptr(), R.data_ptr(), R.data_ptr(), C.data_ptr(),
-                                           side, side, THRD, 1, stream))
+            def mq():
+                _lib.check(L.nklq_quantize_f32(A.data_ptr(), R.data_ptr(), R.data_ptr(), C.data_ptr(),
+                                               rows, cols, THRD, 1, stream))
 
-        def md():
-            _lib.check(L.nklq_dequantize_f32(R.data_ptr(), C.data_ptr(), side, side, THRD, stream))
+            def md():
+                _lib.check(L.nklq_dequantize_f32(R.data_ptr(), C.data_ptr(), rows, cols, THRD, stream))
 
-        for _ in range(5):
-            mq()
-        _, ev = time_region(torch, mq, 50)
-        res["matrix_8192x8192"] = {"fused_GBps": round(BYTES_QUANT * side * side / (ev / 50 * 1e-3) / 1e9, 1)}
-        for _ in range(5):
-            md()
-        _, ev = time_region(torch, md, 50)
-        res["matrix_8192x8192"]["decode_GBps"] = round(BYTES_DEQUANT * side * side / (ev / 50 * 1e-3) / 1e9, 1)
-        del A, R, C
+            for _ in range(5):
+                mq()
+            _, ev = time_region(torch, mq, 30)
+            fq = BYTES_QUANT * tot / (ev / 30 * 1e-3) / 1e9
+            for _ in range(5):
+                md()
+            _, ev2 = time_region(torch, md, 30)
+            fd = BYTES_DEQUANT * tot / (ev2 / 30 * 1e-3) / 1e9
+            res["matrix"][f"{rows}x{cols}"] = {"fused_us": round(ev / 30 * 1e3, 1), "fused_GBps": round(fq, 1),
+                                               "fused_frac_hbm_peak": frac(fq), "decode_us": round(ev2 / 30 * 1e3, 1),
+                                               "decode_GBps": round(fd, 1), "decode_frac_hbm_peak": frac(fd)}
+            del A, R, C
 
     if "multi" in legs:
         # a ResNet-50-shaped list of gradient tensors through the trainer-side buffers
