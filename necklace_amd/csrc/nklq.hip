@@ -24,8 +24,13 @@
 //     path in one extra workgroup of the same launch (codes combined across the
 //     16 lanes of a DPP row);
 //   * 64-bit element indices throughout (vectors of more than 2^31 elements);
-//   * the sum over K payloads (acc_flat_kernel), the matrix form (quant_2d_rows_kernel) and
-//     the many-vectors form (quant_multi_kernel) are described at their kernels.
+//   * a cache line shared by two waves must be completed inside ONE XCD's L2 or it reaches memory
+//     as two partial-line writes: views that start off a 128-byte line, and matrices whose rows
+//     do, get workgroup -> work maps that keep neighbours on one XCD, and the decodes move
+//     their grids onto lines (quant_flat_offline_kernel, deq_flat_shift_kernel, rows_tile_of);
+//   * the sum over K payloads (acc_flat_kernel), the matrix forms (quant_2d_rows_kernel for
+//     wide matrices, quant_bands_kernel for up to 384 columns) and the many-vectors form
+//     (quant_multi_kernel) are described at their kernels.
 //
 // fp32 arithmetic is IEEE: no fast-math, no contraction, denormals kept.
 #include <hip/hip_runtime.h>
@@ -514,12 +519,14 @@ __global__ __launch_bounds__(kAccBlock) void acc_flat_kernel(
 // code, shifted to its bit position, into the tile's 256 words in LDS; after a barrier 256
 // threads store the 1 KiB of words.  When k is not a multiple of 4 (or a base is not 16-byte
 // aligned) rows start at any element: ALIGNED = false issues the same loads with dword
-// alignment, and the last 1-3 columns of a row are moved one by one.
+// alignment, and the last 1-3 columns of a row are moved one by one.  Matrices of up to
+// kBandsMaxColumns columns take the band kernels further down instead.
 constexpr int kRowsBlock = 16 * kWave;  // 1024 threads
 
 // Workgroup -> tile (word row x, column tile T).  Workgroups go to the 8 XCDs round-robin by id; the
 // tiles of one word row are given to ONE XCD, in column order, and 8 neighbouring word rows run
-// side by side on the 8 XCDs.  When rows do not start on cache-line boundaries (k not a multiple
+// side by side on the 8 XCDs (pinned = 1; pinned = 0 is the plain row-major order, used when every
+// row starts on a line).  When rows do not start on cache-line boundaries (k not a multiple
 // of 32) neighbouring tiles of a row share a line at their common edge: written from one XCD the
 // two halves merge in that XCD's L2 into a full-line write, written from two XCDs they reach memory
 // as two partial-line writes.  Returns false for the padding workgroups of the last group of rows.
