@@ -384,24 +384,36 @@ __device__ __forceinline__ uint32_t codes_to_half_tops(uint32_t w)
 // one shift + one mask per TWO elements and one fma per element, against extract + convert + fma
 // per element for an integer multiplier, or two compares + two selects + add for the plain form.
 // Any other t (negative, NaN, infinite, below 2^-125) takes the plain form.
-template <int K, bool ALIGNED, bool MIX>
+// PARTIAL: the last, shorter tile of a vector (rem = 1..1023 elements): the same pass with the words,
+// loads and stores past the end masked (a quad cut by the end goes element by element); the codes of
+// the last word past the end give sums that are never stored.
+template <int K, bool ALIGNED, bool MIX, bool PARTIAL>
 __device__ __forceinline__ void acc_tile(float* o, const PayloadPtrs& pl, int k_payloads, uint64_t word0,
                                          float t, float th, int accumulate, bool divide, float divisor,
-                                         float* my, int lane)
+                                         float* my, int lane, uint32_t rem = kTile)
 {
     constexpr int KMAX = K > 0 ? K : NKLQ_MAX_PAYLOADS_PER_LAUNCH;
     // every payload's word for this lane, all loads in flight together
     uint32_t wd[KMAX];
 #pragma unroll
     for (int p = 0; p < KMAX; ++p)
-        if (K > 0 || p < k_payloads) wd[p] = pl.p[p][word0 + lane];
+        if (K > 0 || p < k_payloads) wd[p] = (!PARTIAL || (uint32_t)lane * 16 < rem) ? pl.p[p][word0 + lane] : 0u;
 
     float s[16];
     if (accumulate) {
         // coalesced read of the running sums, through LDS into the one-word-per-lane layout
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const f32x4 v = ld4<ALIGNED, true>(o + j * 256 + lane * 4);
+            f32x4 v;
+            const uint32_t e = j * 256 + lane * 4;
+            if (!PARTIAL || e + 4 <= rem) {
+                v = ld4<ALIGNED, true>(o + e);
+            } else {
+                v.x = e < rem ? o[e] : 0.0f;
+                v.y = e + 1 < rem ? o[e + 1] : 0.0f;
+                v.z = e + 2 < rem ? o[e + 2] : 0.0f;
+                v.w = 0.0f;
+            }
             *reinterpret_cast<f32x4*>(my + lds_slot(16 * j + (lane >> 2), lane & 3)) = v;
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -456,37 +468,14 @@ __device__ __forceinline__ void acc_tile(float* o, const PayloadPtrs& pl, int k_
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const f32x4 v = *reinterpret_cast<const f32x4*>(my + lds_slot(16 * j + (lane >> 2), lane & 3));
-        st4<ALIGNED, true>(o + j * 256 + lane * 4, v);
-    }
-}
-
-// Fewer than 1024 elements [e0, n) of one vector, bounds-checked: a lane takes elements first,
-// first + step, ... four at a time, so that four loads per payload are in flight instead of one.
-__device__ __forceinline__ void acc_partial_tile(float* acc, const PayloadPtrs& pl, int k_payloads,
-                                                 uint64_t word_offset, uint64_t e0, uint64_t n, float t,
-                                                 int accumulate, bool divide, float divisor, int first,
-                                                 int step)
-{
-    for (uint64_t base = e0 + first; base < n; base += 4 * (uint64_t)step) {
-        uint64_t e[4];
-        float s[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            e[r] = base + (uint64_t)r * step;
-            s[r] = (accumulate && e[r] < n) ? acc[e[r]] : 0.0f;
+        const uint32_t e = j * 256 + lane * 4;
+        if (!PARTIAL || e + 4 <= rem) {
+            st4<ALIGNED, true>(o + e, v);
+        } else {
+            if (e < rem) o[e] = v.x;
+            if (e + 1 < rem) o[e + 1] = v.y;
+            if (e + 2 < rem) o[e + 2] = v.z;
         }
-#pragma unroll 2
-        for (int p = 0; p < k_payloads; ++p) {
-            const uint32_t* words = pl.p[p] + word_offset;
-            uint32_t wd[4];
-#pragma unroll
-            for (int r = 0; r < 4; ++r) wd[r] = e[r] < n ? words[e[r] >> 4] : 0u;
-#pragma unroll
-            for (int r = 0; r < 4; ++r) s[r] = s[r] + deq_code((wd[r] >> (2 * (uint32_t)(e[r] & 15))) & 3u, t);
-        }
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-            if (e[r] < n) acc[e[r]] = divide ? s[r] / divisor : s[r];
     }
 }
 
@@ -496,17 +485,19 @@ __global__ __launch_bounds__(kAccBlock) void acc_flat_kernel(
     uint32_t xs, float t, float th, int accumulate)
 {
     __shared__ __attribute__((aligned(16))) float lds[kAccBlock / kWave][kAccLdsPerWave];
-    if (has_tail && blockIdx.x == gridDim.x - 1) {
-        acc_partial_tile(acc, pl, k_payloads, 0, n_tiles * kTile, n, t, accumulate, false, 1.0f,
-                         threadIdx.x, kAccBlock);
-        return;
-    }
     const int lane = threadIdx.x & (kWave - 1);
     const uint32_t w = threadIdx.x >> 6;
+    if (has_tail && blockIdx.x == gridDim.x - 1) {
+        // the vector's last, shorter tile: one wave of the extra workgroup
+        if (w == 0)
+            acc_tile<K, ALIGNED, MIX, true>(acc + n_tiles * kTile, pl, k_payloads, n_tiles * (kTile / 16), t, th,
+                                            accumulate, false, 1.0f, lds[0], lane, (uint32_t)(n - n_tiles * kTile));
+        return;
+    }
     const uint64_t tile = chunk_of<1, kAccBlock>(blockIdx.x, w, 0, xs);
     if (tile >= n_tiles) return;
-    acc_tile<K, ALIGNED, MIX>(acc + tile * kTile, pl, k_payloads, tile * (kTile / 16), t, th, accumulate,
-                              false, 1.0f, lds[w], lane);
+    acc_tile<K, ALIGNED, MIX, false>(acc + tile * kTile, pl, k_payloads, tile * (kTile / 16), t, th, accumulate,
+                                     false, 1.0f, lds[w], lane);
 }
 
 // ---------------------------------------------------------------- matrix (n, k) kernels
@@ -922,13 +913,13 @@ __global__ __launch_bounds__(kAccBlock) void acc_multi_kernel(AccSegments seg, P
     const uint64_t n = seg.n[sidx];
     const uint64_t e0 = (uint64_t)(q - seg.first[sidx]) * kTile;
     if (e0 + kTile > n) {
-        // last, partial tile of the vector
-        acc_partial_tile(seg.acc[sidx], pl, k_payloads, seg.word_offset[sidx], e0, n, t, accumulate,
-                         divide, divisor, lane, kWave);
+        // last, shorter tile of the vector
+        acc_tile<K, ALIGNED, MIX, true>(seg.acc[sidx] + e0, pl, k_payloads, seg.word_offset[sidx] + (e0 >> 4), t,
+                                        th, accumulate, divide, divisor, lds[w], lane, (uint32_t)(n - e0));
         return;
     }
-    acc_tile<K, ALIGNED, MIX>(seg.acc[sidx] + e0, pl, k_payloads, seg.word_offset[sidx] + (e0 >> 4), t, th,
-                              accumulate, divide, divisor, lds[w], lane);
+    acc_tile<K, ALIGNED, MIX, false>(seg.acc[sidx] + e0, pl, k_payloads, seg.word_offset[sidx] + (e0 >> 4), t, th,
+                                     accumulate, divide, divisor, lds[w], lane);
 }
 
 // ---------------------------------------------------------------- copy (measurement aid)
