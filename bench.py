@@ -50,7 +50,7 @@ def parse():
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="CPU-baseline time budget; 0 skips it")
     ap.add_argument("--legs", default="deq,acc,configs,wrapper,copy,cpu",
                     help="extra legs after the timed quantize steps: deq, acc, configs, wrapper, copy, cpu, "
-                         "and (off by default) matrix, multi (comma list, '' = none)")
+                         "and (off by default) matrix, multi, accsweep (comma list, '' = none)")
     return ap.parse_args()
 
 
@@ -547,6 +547,26 @@ def main():
 
     if "wrapper" in legs:
         bench_wrapper(torch, L, _lib, stream, res)
+
+    if "accsweep" in legs:
+        # the fixed-order sum against the number of payloads, at gradient size: where the payloads stop
+        # fitting the 256 MB memory-side cache (K >= 4 here) the time per payload jumps
+        import ctypes as ct
+        wl = _lib.packed_words(n)
+        big = torch.randint(-2 ** 31, 2 ** 31 - 1, (16, wl), dtype=torch.int32, device="cuda", generator=gen)
+        accl = torch.empty(n, dtype=torch.float32, device="cuda")
+        ptrl = (ct.c_void_p * 16)(*[big[p].data_ptr() for p in range(16)])
+        res["dequant_accumulate_by_payloads"] = {}
+        for kp in (1, 2, 3, 4, 6, 8, 12, 16):
+            f = lambda: _lib.check(L.nklq_dequant_accumulate_f32(accl.data_ptr(), ptrl, kp, n, THRD, 0, stream))
+            for _ in range(10):
+                f()
+            _, ev = time_region(torch, f, 20)
+            gb = (0.25 * kp + 4) * n / (ev / 20 * 1e-3) / 1e9
+            res["dequant_accumulate_by_payloads"][str(kp)] = {
+                "us": round(ev / 20 * 1e3, 1), "GBps": round(gb, 1), "frac_hbm_peak": frac(gb),
+                "payload_MB": round(4 * wl * kp / 1e6)}
+        del big, accl
 
     if "matrix" in legs:
         # the reference's own layout: (n, k) matrix, codes packed down the columns; wide and narrow,
