@@ -118,6 +118,8 @@ def cpu_baseline(g_slab, r_slab, budget_s, thrd=THRD):
                   f"({el:.1f} s, C restatement of necklace/cuda/quantize.py, OpenMP {threads} threads)",
         "one_thread_GBps": round(BYTES_QUANT * n * reps1 / el1 / 1e9, 3),
         "numpy_one_thread_GBps": round(BYTES_QUANT * m * repsn / eln / 1e9, 3),
+        # the reference's own CPU route would be numba's CUDA simulator; it is used only if it is there
+        "numba_installed": __import__("importlib.util").util.find_spec("numba") is not None,
     }
 
 
@@ -298,11 +300,15 @@ def bench_configs(torch, L, _lib, stream, gen, res, cpu_seconds):
         r5.zero_()
         _, ev = time_region(torch, step5, steps5)
         ms = ev / steps5
+        slab5 = g5[:1 << 26].cpu().numpy() if cpu_seconds > 0 else None
         res["config5"] = {"elements": n5, "chunk": chunk5, "launches_per_step": len(pieces), "steps": steps5,
                           "ms_per_step": round(ms, 4), "GBps": round(BYTES_QUANT * n5 / ms / 1e6, 1),
                           "frac_hbm_peak": frac(BYTES_QUANT * n5 / ms / 1e6), "elements_per_s": round(n5 / ms * 1e3),
                           "resident_GB": round((2 * 4 * n5 + 4 * _lib.packed_words(n5)) / 1e9, 2)}
         del g5, r5, c5
+        if slab5 is not None:
+            res["config5"]["cpu_baseline"] = cpu_baseline_small(slab5, np.zeros(1 << 26, np.float32), t5, cpu_seconds * 0.2,
+                                                                "a 67,108,864-element slice of config 5")
     else:
         res["config5"] = {"skipped": f"only {free / 1e9:.0f} GB of HBM free"}
 
