@@ -689,6 +689,16 @@ __device__ __forceinline__ void band_row_col(uint32_t li, uint32_t k, uint32_t i
     *col = li - q * k;
 }
 
+// Workgroup -> range.  A range rarely starts on a 128-byte line, so neighbouring ranges share one:
+// ranges are dealt to the XCDs in runs of kBandRun (workgroup b runs on XCD b % 8), so that all but
+// one shared line in kBandRun is completed inside one XCD's L2.
+constexpr uint32_t kBandRun = 8;
+__device__ __forceinline__ uint64_t band_range_of(uint32_t b)
+{
+    const uint32_t xcd = b & 7u, j = b >> 3;
+    return ((uint64_t)(j / kBandRun) * 8 + xcd) * kBandRun + (j % kBandRun);
+}
+
 template <bool ADD, bool NT, bool ALIGNED>
 __global__ __launch_bounds__(kBandsBlock) void quant_bands_kernel(
     const float* g, const float* rin, float* rout, uint32_t* __restrict__ c, uint64_t n, uint32_t k,
@@ -696,7 +706,8 @@ __global__ __launch_bounds__(kBandsBlock) void quant_bands_kernel(
 {
     __shared__ uint32_t words[kBandsMaxColumns];
     const uint64_t m = (n + 15) / 16;
-    const uint64_t x0 = (uint64_t)blockIdx.x * bands_per_wg;
+    const uint64_t x0 = band_range_of(blockIdx.x) * bands_per_wg;
+    if (x0 >= m) return;  // padding workgroups of the last group of runs
     const uint64_t x1 = (x0 + bands_per_wg < m) ? x0 + bands_per_wg : m;
     const uint64_t e0 = x0 * 16 * k;
     const uint64_t e1 = (x1 * 16 < n ? x1 * 16 : n) * k;
@@ -777,7 +788,7 @@ __global__ __launch_bounds__(kBandsBlock) void deq_bands_kernel(
 {
     __shared__ uint32_t words[kBandsMaxColumns];
     const uint64_t m = (n + 15) / 16;
-    const uint64_t x0 = (uint64_t)blockIdx.x * bands_per_wg;
+    const uint64_t x0 = (uint64_t)blockIdx.x * bands_per_wg;  // (runs per XCD measured slower for the decode)
     const uint64_t x1 = (x0 + bands_per_wg < m) ? x0 + bands_per_wg : m;
     const uint64_t e0 = x0 * 16 * k;
     const uint64_t e1 = (x1 * 16 < n ? x1 * 16 : n) * k;
@@ -1310,12 +1321,13 @@ int launch_acc_multi(const AccSegments& seg, const PayloadPtrs& pl, int k, bool 
 }
 
 // Bands per workgroup of the band kernels, and the launch's workgroup count (0: out of range).
-uint32_t bands_grid(uint64_t n_rows, uint64_t n_cols, uint64_t range, uint32_t* bands_per_wg)
+uint32_t bands_grid(uint64_t n_rows, uint64_t n_cols, uint64_t range, bool runs, uint32_t* bands_per_wg)
 {
     const uint64_t m = n_rows / 16 + (n_rows % 16 ? 1 : 0);
     const uint64_t per = range / (16 * n_cols);
     *bands_per_wg = (uint32_t)(per ? per : 1);
-    const uint64_t blocks = (m + *bands_per_wg - 1) / *bands_per_wg;
+    const uint64_t ranges = (m + *bands_per_wg - 1) / *bands_per_wg;
+    const uint64_t blocks = runs ? (ranges + 8 * kBandRun - 1) / (8 * kBandRun) * (8 * kBandRun) : ranges;  // whole groups of runs
     return blocks > 0x7FFFFFFFull ? 0u : (uint32_t)blocks;
 }
 
@@ -1404,7 +1416,7 @@ int nklq_quantize_f32(const float* g, const float* r_in, float* r_out, uint32_t*
     const uint64_t m = n_rows / 16 + (n_rows % 16 ? 1 : 0);
     if (n_cols <= kBandsMaxColumns) {
         uint32_t per;
-        const uint32_t grid = bands_grid(n_rows, n_cols, kBandsRangeQuant, &per);
+        const uint32_t grid = bands_grid(n_rows, n_cols, kBandsRangeQuant, true, &per);
         if (grid == 0) return NKLQ_ERANGE;
         const uint32_t k32 = (uint32_t)n_cols;
         const uint32_t inv = (uint32_t)(0x100000000ull / k32) + 1u;
@@ -1475,7 +1487,7 @@ int nklq_dequantize_f32(float* out, const uint32_t* c, uint64_t n_rows, uint64_t
     const uint64_t m = n_rows / 16 + (n_rows % 16 ? 1 : 0);
     if (n_cols <= kBandsMaxColumns) {
         uint32_t per;
-        const uint32_t grid = bands_grid(n_rows, n_cols, kBandsRangeDecode, &per);
+        const uint32_t grid = bands_grid(n_rows, n_cols, kBandsRangeDecode, false, &per);
         if (grid == 0) return NKLQ_ERANGE;
         const uint32_t k32 = (uint32_t)n_cols;
         const uint32_t inv = (uint32_t)(0x100000000ull / k32) + 1u;
