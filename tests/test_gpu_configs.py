@@ -168,3 +168,24 @@ def test_config5_hbm_sizing_chunked_error_feedback():
             assert torch.equal(r_whole.view(torch.int32), r.view(torch.int32))
             del r_whole, c_whole
     assert int((c != 0).sum()) > 0
+
+
+@pytest.mark.parametrize("n,k", [(4099, 8191), (1_000_003, 17), (100_003, 384), (50_001, 385), (2_000_001, 3)])
+def test_large_matrices_every_kernel_regime_against_the_oracle(n, k):
+    """Tens of millions of elements per shape: many workgroups per XCD, padded grids (word rows in
+    groups of 8, band ranges in runs), rows off 128-byte lines; fused step with a residual, then the
+    decode of the words into the same buffer."""
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(n + k)
+    thrd = 2e-3
+    A = torch.randn(n, k, device="cuda", generator=gen) * 1e-3
+    R = torch.randn(n, k, device="cuda", generator=gen) * 1e-3
+    C = torch.full(((n + 15) // 16, k), -1, dtype=torch.int32, device="cuda")
+    a_host, r_host = A.cpu().numpy(), R.cpu().numpy()
+    q.cu_fn_matrix_quantize_e(A, C, R, thrd, add_residual=True)
+    want_c, want_r = oracle.c.quantize(a_host, thrd, R_in=r_host)
+    assert_words_equal(C.cpu().numpy().view(np.uint32), want_c, f"{n}x{k} codes")
+    assert_bits_equal(R.cpu().numpy(), want_r, f"{n}x{k} residual")
+    del a_host, r_host, want_r
+    q.cu_fn_matrix_dequantize_e(R, C, None, thrd)
+    assert_bits_equal(R.cpu().numpy(), oracle.c.dequantize(want_c, n, thrd), f"{n}x{k} decode")
