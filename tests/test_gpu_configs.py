@@ -189,3 +189,28 @@ def test_large_matrices_every_kernel_regime_against_the_oracle(n, k):
     del a_host, r_host, want_r
     q.cu_fn_matrix_dequantize_e(R, C, None, thrd)
     assert_bits_equal(R.cpu().numpy(), oracle.c.dequantize(want_c, n, thrd), f"{n}x{k} decode")
+
+
+@pytest.mark.parametrize("og,orr,oo", [(1, 1, 1), (0, 3, 31), (4, 4, 8), (16, 0, 16), (0, 16, 5)])
+def test_large_flat_views_off_cache_lines(og, orr, oo):
+    """20 M elements cut out of larger buffers at element offsets: the residual (and the decode
+    target) start off a 128-byte line, which takes the run-dealt quantize and the line-shifted
+    decode; the guard elements around the views must stay untouched."""
+    n, thrd = 20_000_003, 2e-3
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(og * 100 + orr * 10 + oo)
+    gbuf = torch.randn(n + 64, device="cuda", generator=gen) * 1e-3
+    rbuf = torch.randn(n + 64, device="cuda", generator=gen) * 1e-3
+    obuf = torch.full((n + 64,), 9.0, device="cuda")
+    g, r, out = gbuf[og:og + n], rbuf[orr:orr + n], obuf[oo:oo + n]
+    g_host, r_host = g.cpu().numpy(), r.cpu().numpy()
+    guard_lo, guard_hi = rbuf[:orr].clone(), rbuf[orr + n:].clone()
+    C = words_like(n)
+    q.cu_fn_matrix_quantize_e(g, C, r, thrd, add_residual=True)
+    want_c, want_r = oracle.c.quantize(g_host, thrd, R_in=r_host)
+    assert_words_equal(host_words(C), want_c, "codes")
+    assert_bits_equal(r.cpu().numpy(), want_r, "residual")
+    assert torch.equal(rbuf[:orr], guard_lo) and torch.equal(rbuf[orr + n:], guard_hi)
+    q.cu_fn_matrix_dequantize_e(out, C, None, thrd)
+    assert_bits_equal(out.cpu().numpy(), oracle.c.dequantize(want_c, n, thrd), "decode")
+    assert float(obuf[:oo].sum()) == 9.0 * oo and float(obuf[oo + n:].sum()) == 9.0 * (64 - oo)
