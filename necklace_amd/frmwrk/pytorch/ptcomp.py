@@ -434,7 +434,7 @@ def _cfg_for_params(params, kn, cfg):
     sig = ("params", tuple((i, p.numel()) for i, p in zip(ids, params)), kn)
     if cfg.get("_signature") != sig:
         old_gc, old_ids = cfg.get("compressor"), cfg.get("_ids", [])
-        dev = next((p.device for p in params if p.is_cuda), torch.device("cuda"))
+        dev = params[0].device if params else torch.device("cuda")
         built = init_grad_comp_cfg(params, kn, cfg, device=dev, rank=cfg.get("rank", 0))
         _carry_residuals(old_gc if cfg.get("_signature", ("",))[0] == "params" else None, old_ids,
                          built["compressor"], ids)

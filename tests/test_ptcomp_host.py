@@ -65,3 +65,45 @@ def test_state_round_trip():
     assert torch.equal(gc2.resi, gc.resi)
     with pytest.raises(ValueError):
         ptcomp.GradCompressor([2001], kn=1, device="cpu").load_state_dict(st)
+
+
+def test_bucketing_follows_the_reference_rule():
+    """Consecutive tensors, a new bucket when the next one would pass the limit, an oversized tensor
+    alone (the shape of _take_tensors at necklace/frmwrk/pytorch/ptprms.py:258)."""
+    ts = [torch.zeros(n) for n in (100, 200, 300, 1000, 50, 60)]
+    sizes = lambda bs: [[t.numel() for t in b] for b in bs]
+    assert sizes(ptcomp._take_buckets(ts, 4 * 600)) == [[100, 200, 300], [1000], [50, 60]]
+    assert sizes(ptcomp._take_buckets(ts, 4 * 10 ** 6)) == [[100, 200, 300, 1000, 50, 60]]
+    assert sizes(ptcomp._take_buckets(ts, 1)) == [[100], [200], [300], [1000], [50], [60]]
+    assert ptcomp._take_buckets([], 1024) == []
+
+
+def test_layout_is_rebuilt_when_the_optimizer_changes_and_residuals_move_along():
+    a, b = torch.nn.Parameter(torch.zeros(3000)), torch.nn.Parameter(torch.zeros(500))
+    cfg = {"grad_comp_threshold": 0.25, "grad_size_threshold": 1001}
+    gc1 = ptcomp._cfg_for_params([a, b], 2, cfg)
+    assert gc1.grd_cmps == [True, False] and ptcomp._cfg_for_params([a, b], 2, cfg) is gc1  # kept while nothing changes
+    gc1.grd_resi[0].copy_(torch.arange(3000, dtype=torch.float32))
+    d = torch.nn.Parameter(torch.zeros(2000))
+    gc2 = ptcomp._cfg_for_params([a, b, d], 2, cfg)
+    assert gc2 is not gc1 and gc2.grd_cmps == [True, False, True]
+    assert torch.equal(gc2.grd_resi[0], torch.arange(3000, dtype=torch.float32))  # what a is owed survives
+    assert float(gc2.grd_resi[2].abs().sum()) == 0.0
+    assert cfg["compressor"] is gc2 and cfg["grad_comp_threshold"] == 0.25
+
+
+def test_small_gradients_need_a_collective_when_there_are_several_workers():
+    g = [torch.ones(10), torch.ones(20)]
+    ptcomp._reduce_small(g, 1, None, True)            # one worker: nothing to do
+    with pytest.raises(ValueError):
+        ptcomp._reduce_small(g, 2, None, True)
+    seen = []
+
+    def allreduce(flat):
+        seen.append(flat.numel())
+        flat.mul_(2.0)                                # a second worker with the same values
+
+    ptcomp._reduce_small(g, 2, allreduce, True)
+    assert seen == [30] and all(float(t.sum()) == t.numel() for t in g)   # (1 + 1) / 2
+    ptcomp._reduce_small(g, 2, allreduce, False)
+    assert all(float(t.sum()) == 2 * t.numel() for t in g)                # the reduce form: summed, not averaged
