@@ -254,6 +254,27 @@ def test_accumulate_and_decode_with_unusual_thresholds(thrd):
     assert_bits_equal(gpu_dequantize(pl[0], n, thrd), oracle.c.dequantize(pl[0], n, thrd), f"decode thrd={thrd}")
 
 
+@pytest.mark.parametrize("tbits", [0x00800000, 0x00FFFFFF, 0x01000000, 0x01000001, 0x03800000, 0x7E7FFFFF, 0x7F000000, 0x7F7FFFFF])
+def test_accumulate_at_the_ends_of_the_exponent_range(tbits):
+    """Thresholds around the smallest normal numbers (t/2 exact or not: that decides between the
+    fused multiply-add form and the compare-and-select form) and the largest finite ones, with
+    running sums of the threshold's own magnitude: results that are denormal, cancel to zero or
+    overflow must carry the same bits as a plain left-to-right fp32 sum."""
+    t = float(np.array([tbits], dtype=np.uint32).view(np.float32)[0])
+    rng = np.random.default_rng(tbits & 0xFFFF)
+    n = 4096 + 37
+    pl = [pack_codes_np(rng.integers(0, 4, size=n).astype(np.uint32), n) for _ in range(6)]
+    with np.errstate(over="ignore"):
+        base = (rng.uniform(-3, 3, n) * t).astype(np.float32)      # a few thresholds away from zero
+    base[::5] = (rng.integers(-3, 4, size=len(base[::5])) * np.float32(t)).astype(np.float32) if t < 1e38 else base[::5]
+    for acc0 in (None, base):
+        with np.errstate(invalid="ignore", over="ignore"):
+            want = oracle.c.dequant_accumulate(pl, n, t, acc=None if acc0 is None else acc0.copy())
+        acc = torch.full((n,), 5.0, device="cuda") if acc0 is None else dev(acc0)
+        q.cu_fn_dequantize_accumulate_e(acc, [dev(w) for w in pl], t, accumulate=acc0 is not None)
+        assert_bits_equal(acc.cpu().numpy(), want, f"t=0x{tbits:08X} accumulate={acc0 is not None}")
+
+
 def test_accumulate_keeps_signed_zero_like_the_reference():
     """-0.0 + (+0.0) is +0.0: an all-zero payload turns a -0.0 running sum into +0.0, on both sides."""
     n = 2048 + 3
