@@ -525,6 +525,32 @@ def main():
             "note": "50 MB working set: served by the 256 MB memory-side cache when repeated",
         }
         del payloads, acc
+        # the size necklace reduces at a time: one 256 MB bucket (nccl_reduce_bucket_size,
+        # necklace/frmwrk/pytorch/ptprms.py:253) = 67,108,864 elements, 8 payloads of 16 MB that another
+        # kernel has just written (as an all-gather would have) before every sum; only the sums are timed
+        nk = 1 << 26
+        wk = _lib.packed_words(nk)
+        arrived = torch.randint(-2 ** 31, 2 ** 31 - 1, (K_PAYLOADS, wk), dtype=torch.int32, device="cuda", generator=gen)
+        inbox = torch.empty_like(arrived)
+        acck = torch.empty(nk, dtype=torch.float32, device="cuda")
+        ptrk = (ct.c_void_p * K_PAYLOADS)(*[inbox[p].data_ptr() for p in range(K_PAYLOADS)])
+        pairs_k = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(30)]
+        for i in range(40):
+            inbox.copy_(arrived)
+            if i >= 10:
+                pairs_k[i - 10][0].record()
+            _lib.check(L.nklq_dequant_accumulate_f32(acck.data_ptr(), ptrk, K_PAYLOADS, nk, THRD, 0, stream))
+            if i >= 10:
+                pairs_k[i - 10][1].record()
+        torch.cuda.synchronize()
+        tk_ms = sorted(a.elapsed_time(b) for a, b in pairs_k)[len(pairs_k) // 2]
+        gbk = (0.25 * K_PAYLOADS + 4) * nk / (tk_ms * 1e-3) / 1e9
+        res["dequant_accumulate_256MB_bucket"] = {
+            "payloads": K_PAYLOADS, "elements": nk, "elements_per_s": round(nk / (tk_ms * 1e-3)),
+            "ms": round(tk_ms, 4), "GBps": round(gbk, 1), "frac_hbm_peak": frac(gbk),
+            "note": "median of 30 sums, each right after its 128 MB of payloads were written",
+        }
+        del arrived, inbox, acck
         # the same sum at gradient size: 8 random payloads (the kernel's time does not depend on the codes)
         if n >= 1 << 24:
             wl = _lib.packed_words(n)
