@@ -122,6 +122,9 @@ class GradCompressor:
         # parameters that have a gradient)
         self._idx = [i for i, c in enumerate(self.grd_cmps) if c]
         self._live_key, self._live_tabs = None, None
+        # what Tensor.get_device() returns for tensors that live where the buffers do; host tensors
+        # (-1) never match: there is no CPU path
+        self._dev_index = self.resi.get_device() if self.resi.is_cuda else -2
         self._pl_arr = (ct.c_void_p * self.kn)(*[self.recv[k].data_ptr() for k in range(self.kn)])
 
     def _tables(self, tensors, what):
@@ -129,6 +132,32 @@ class GradCompressor:
         call; cached while the same subset comes back.  Returns (count, ptrs, r, c, n, word_offset)."""
         if len(tensors) != len(self.layout):
             raise ValueError(f"expected {len(self.layout)} {what}s, got {len(tensors)}")
+        # one pass over the tensors (this runs every step, for every parameter); what exactly is
+        # wrong is worked out only when something is
+        live, addrs = [], []
+        numels, f32, dev_index = self.layout.numels, torch.float32, self._dev_index
+        for i in self._idx:
+            t = tensors[i]
+            if t is None:
+                continue
+            if (t.numel() != numels[i] or t.dtype is not f32 or t.get_device() != dev_index
+                    or not t.is_contiguous()):
+                self._refuse(tensors, what)
+            live.append(i)
+            addrs.append(t.data_ptr())
+        key = tuple(live)
+        if key != self._live_key:
+            m = len(live)
+            self._live_key = key
+            self._live_tabs = (
+                (ct.c_void_p * m)(*[self.grd_resi[i].data_ptr() for i in live]),
+                (ct.c_void_p * m)(*[self.grd_comp[i].data_ptr() for i in live]),
+                (ct.c_uint64 * m)(*[self.layout.numels[i] for i in live]),
+                (ct.c_uint64 * m)(*[self.layout.word_offset[i] for i in live]))
+        return (len(live), (ct.c_void_p * len(live))(*addrs)) + self._live_tabs
+
+    def _refuse(self, tensors, what):
+        """Raise for the first tensor that does not fit: sizes first, then type, layout, device."""
         live = [i for i in self._idx if tensors[i] is not None]
         for i in live:
             if tensors[i].numel() != self.layout.numels[i]:
@@ -142,17 +171,7 @@ class GradCompressor:
                 raise ValueError(f"{what} {i} must be contiguous")
             if t.device != self.resi.device:
                 raise ValueError(f"{what} {i} is on {t.device}, the buffers are on {self.resi.device}")
-        key = tuple(live)
-        if key != self._live_key:
-            m = len(live)
-            self._live_key = key
-            self._live_tabs = (
-                (ct.c_void_p * m)(*[self.grd_resi[i].data_ptr() for i in live]),
-                (ct.c_void_p * m)(*[self.grd_comp[i].data_ptr() for i in live]),
-                (ct.c_uint64 * m)(*[self.layout.numels[i] for i in live]),
-                (ct.c_uint64 * m)(*[self.layout.word_offset[i] for i in live]))
-        ptrs = (ct.c_void_p * len(live))(*[tensors[i].data_ptr() for i in live])
-        return (len(live), ptrs) + self._live_tabs
+        raise AssertionError("unreachable: the quick check and the detailed one disagree")
 
     # ---- send side
 
