@@ -376,7 +376,7 @@ def load_grad_comp_state(grad_comp_cfg, state):
 
 # --------------------------------------------------------------------------- ptprms call surface
 #
-# Same names, argument order and return value (None) as necklace/frmwrk/pytorch/ptprms.py:319-401, so
+# Same names, argument order and return value (None) as necklace/frmwrk/pytorch/ptprms.py:300-401, so
 # that a trainer can import them from here instead.  What differs is what travels:
 #
 #   nc             where necklace passes its NCCL communicator.  Collectives are not part of this
@@ -527,9 +527,12 @@ def _reduce_buckets_form(nc, kn, root, params, cfg):
 
 
 def _reduce_opt(nc, kn, root, opt, grad_comp_cfg):
+    _reduce_params(nc, kn, root, _opt_params(opt), grad_comp_cfg)
+
+
+def _reduce_params(nc, kn, root, params, grad_comp_cfg):
     if grad_comp_cfg is None:
         raise ValueError("grad_comp_cfg is required: this is the compressed path")
-    params = _opt_params(opt)
     form = grad_comp_cfg.get("form", "params")
     if form == "params":
         _reduce_params_form(nc, kn, root, params, grad_comp_cfg)
@@ -546,6 +549,18 @@ def _per_optimizer(opt, grad_comp_cfg):
         raise ValueError("several optimizers need one grad_comp_cfg each (their residuals differ)")
     cfgs = grad_comp_cfg if isinstance(grad_comp_cfg, (list, tuple)) else [grad_comp_cfg] * len(opt)
     return list(zip(opt, cfgs))
+
+
+def grads_do_nccl_allreduce(nc, kn, model, prm_revs=None, grad_comp_cfg=None):
+    """Compressed counterpart of ptprms.grads_do_nccl_allreduce
+    (necklace/frmwrk/pytorch/ptprms.py:300-315): the same step over a model's trainable parameters
+    instead of an optimizer's.  Returns None."""
+    params = [p for p in model.parameters() if p.requires_grad]
+    for p in params:
+        if p.grad is not None and p.grad.requires_grad:
+            # the reference's wording (ptprms.py:307-310)
+            raise RuntimeError("DistributedDataParallel only works with gradients that don't require grad")
+    _reduce_params(nc, kn, None, params, grad_comp_cfg)
 
 
 def opt_one_grads_do_nccl_allreduce(nc, kn, opt, prm_revs=None, grad_comp_cfg=None):

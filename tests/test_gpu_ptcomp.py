@@ -216,6 +216,33 @@ def test_ptprms_call_surface_on_a_real_optimizer():
     assert int((cfg1["compressor"].comp != 0).sum()) > 0
 
 
+def test_model_form_gives_what_the_optimizer_form_gives():
+    """grads_do_nccl_allreduce(nc, kn, model, ...) (necklace/frmwrk/pytorch/ptprms.py:300-315) walks
+    model.parameters() instead of an optimizer's groups; frozen parameters are left out."""
+    thrd, kn = 1e-3, 2
+    cfg_a = {"grad_comp_threshold": thrd, "grad_size_threshold": 1001}
+    cfg_b = dict(cfg_a)
+    model_a, opt_a, _, _ = _mlp_with_grads(seed=5)
+    model_b, _, _, _ = _mlp_with_grads(seed=5)
+    ptcomp.opt_grads_do_nccl_allreduce(TwoWorkersWithEqualData(), kn, opt_a, None, grad_comp_cfg=cfg_a)
+    assert ptcomp.grads_do_nccl_allreduce(TwoWorkersWithEqualData(), kn, model_b, None, grad_comp_cfg=cfg_b) is None
+    torch.cuda.synchronize()
+    for pa, pb in zip(model_a.parameters(), model_b.parameters()):
+        assert torch.equal(pa.grad, pb.grad)
+    # a frozen parameter is not part of the layout, its stale gradient is left alone
+    model_c, _, _, _ = _mlp_with_grads(seed=5)
+    first = next(model_c.parameters())
+    first.requires_grad_(False)
+    stale = first.grad.clone()
+    cfg_c = dict(cfg_a)
+    ptcomp.grads_do_nccl_allreduce(TwoWorkersWithEqualData(), kn, model_c, None, grad_comp_cfg=cfg_c)
+    torch.cuda.synchronize()
+    assert torch.equal(first.grad, stale)
+    assert len(cfg_c["compressor"].layout) == len(list(model_c.parameters())) - 1
+    for pa, pc in list(zip(model_a.parameters(), model_c.parameters()))[1:]:
+        assert torch.equal(pa.grad, pc.grad)
+
+
 def test_a_gradient_that_first_appears_at_step_two_and_a_parameter_added_later():
     """The layout covers all parameters of the optimizer from the start, so one whose .grad is None
     at step 1 simply joins at step 2 with a zero residual; a parameter group added later rebuilds

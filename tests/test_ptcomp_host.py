@@ -107,3 +107,14 @@ def test_small_gradients_need_a_collective_when_there_are_several_workers():
     assert seen == [30] and all(float(t.sum()) == t.numel() for t in g)   # (1 + 1) / 2
     ptcomp._reduce_small(g, 2, allreduce, False)
     assert all(float(t.sum()) == 2 * t.numel() for t in g)                # the reduce form: summed, not averaged
+
+
+def test_model_form_refuses_a_gradient_that_requires_grad():
+    """As necklace/frmwrk/pytorch/ptprms.py:307-310 does, before anything is laid out."""
+    model = torch.nn.Linear(4, 3)
+    model.weight.grad = torch.zeros(3, 4, requires_grad=True)
+    with pytest.raises(RuntimeError):
+        ptcomp.grads_do_nccl_allreduce(None, 1, model, None, grad_comp_cfg={})
+    model.weight.grad = torch.zeros(3, 4)
+    with pytest.raises(ValueError):  # the compressed path needs its configuration
+        ptcomp.grads_do_nccl_allreduce(None, 1, model, None, grad_comp_cfg=None)
