@@ -96,3 +96,56 @@ def test_accumulate_random_counts_lengths_offsets(seed):
             what = f"seed={seed} n={n} K={K} thrd={thrd} off={off} accumulate={acc0}"
             assert_bits_equal(acc.cpu().numpy(), want, what)
             assert float(buf[:off].sum()) == 2.0 * off and float(buf[off + n:].sum()) == 2.0 * (16 - off), what
+
+
+@pytest.mark.parametrize("seed", range(3))
+def test_many_vectors_random_lists(seed):
+    """The many-vectors entry points on random lists (1 to 230 vectors of 1 to 200,000 elements,
+    random gaps between them inside one arena, 1 to 9 messages): every vector equals its own flat
+    result and nothing between the vectors is written."""
+    rng = np.random.default_rng(4000 + seed)
+    for _ in range(4):
+        count = int(rng.choice([rng.integers(1, 10), rng.integers(10, 97), rng.integers(97, 230)]))
+        ns = [int(rng.choice([rng.integers(1, 300), rng.integers(300, 5000), rng.integers(5000, 200000)]))
+              for _ in range(count)]
+        thrd, K = float(rng.choice([1e-3, 2e-3, 0.5])), int(rng.integers(1, 10))
+        fused, acc0 = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+        divisor = float(rng.choice([1.0, K, 3.0]))
+        what = f"seed={seed} count={count} total={sum(ns)} thrd={thrd} K={K} fused={fused} acc0={acc0} / {divisor}"
+        gaps = rng.integers(1, 9, size=count)
+        starts = np.cumsum([4] + [n + int(g) for n, g in zip(ns, gaps)])[:-1]
+        size = int(starts[-1]) + ns[-1] + 8
+        between = np.ones(size, bool)
+        for s, n in zip(starts, ns):
+            between[s:s + n] = False
+        a, r0 = _values(rng, size, thrd), _values(rng, size, thrd * 0.5)
+        r0[between] = 5.0
+        g_arena, r_arena = dev(a), dev(r0)
+        wn = [(n + 15) // 16 for n in ns]
+        woffs = [int(w) for w in np.cumsum([0] + wn)[:-1]]
+        total_words = sum(wn)
+        msgs = rng.integers(0, 2 ** 32, size=(K, total_words + 4), dtype=np.uint64).astype(np.uint32)
+        recv = dev(msgs)
+        q.cu_fn_quantize_multi_e([g_arena[s:s + n] for s, n in zip(starts, ns)],
+                                 [recv[0, w:w + m] for w, m in zip(woffs, wn)],
+                                 [r_arena[s:s + n] for s, n in zip(starts, ns)], thrd, add_residual=fused)
+        got_r, got_w = r_arena.cpu().numpy(), host_words(recv)
+        for i, (s, n) in enumerate(zip(starts, ns)):
+            want_c, want_r = oracle.c.quantize(a[s:s + n], thrd, R_in=r0[s:s + n] if fused else None)
+            assert_words_equal(got_w[0, woffs[i]:woffs[i] + wn[i]], want_c, f"{what}: vector {i} n={n}")
+            assert_bits_equal(got_r[s:s + n], want_r, f"{what}: vector {i} n={n}")
+        assert (got_r[between] == 5.0).all(), what
+        assert np.array_equal(got_w[0, total_words:], msgs[0, total_words:]) and np.array_equal(got_w[1:], msgs[1:]), what
+        base = _values(rng, size, thrd)
+        base[between] = 9.0
+        o_arena = dev(base)
+        q.cu_fn_dequantize_accumulate_multi_e([o_arena[s:s + n] for s, n in zip(starts, ns)], woffs, recv, thrd,
+                                              accumulate=acc0, divisor=divisor)
+        got = o_arena.cpu().numpy()
+        for i, (s, n) in enumerate(zip(starts, ns)):
+            want = oracle.c.dequant_accumulate([got_w[k, woffs[i]:woffs[i] + wn[i]] for k in range(K)], n, thrd,
+                                               acc=base[s:s + n] if acc0 else None)
+            if divisor != 1.0:
+                want = (want / np.float32(divisor)).astype(np.float32)
+            assert_bits_equal(got[s:s + n], want, f"{what}: sum of vector {i} n={n}")
+        assert (got[between] == 9.0).all(), what
