@@ -389,7 +389,7 @@ __device__ __forceinline__ uint32_t codes_to_half_tops(uint32_t w)
 // the last word past the end give sums that are never stored.
 template <int K, bool ALIGNED, bool MIX, bool PARTIAL>
 __device__ __forceinline__ void acc_tile(float* o, const PayloadPtrs& pl, int k_payloads, uint64_t word0,
-                                         float t, float th, int accumulate, bool divide, float divisor,
+                                         float t, float th, int accumulate, float divisor, float recip,
                                          float* my, int lane, uint32_t rem = kTile)
 {
     constexpr int KMAX = K > 0 ? K : NKLQ_MAX_PAYLOADS_PER_LAUNCH;
@@ -450,7 +450,12 @@ __device__ __forceinline__ void acc_tile(float* o, const PayloadPtrs& pl, int k_
             }
         }
     }
-    if (divide) {  // IEEE division, correctly rounded (not a reciprocal)
+    if (recip != 0.0f) {
+        // the divisor is a power of two: its reciprocal is exact, so the product is the same real
+        // number as the quotient and rounds to the same bits (one multiply instead of ~10 instructions)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[i] = s[i] * recip;
+    } else if (divisor != 1.0f) {  // IEEE division, correctly rounded
 #pragma unroll
         for (int i = 0; i < 16; ++i) s[i] = s[i] / divisor;
     }
@@ -491,13 +496,13 @@ __global__ __launch_bounds__(kAccBlock) void acc_flat_kernel(
         // the vector's last, shorter tile: one wave of the extra workgroup
         if (w == 0)
             acc_tile<K, ALIGNED, MIX, true>(acc + n_tiles * kTile, pl, k_payloads, n_tiles * (kTile / 16), t, th,
-                                            accumulate, false, 1.0f, lds[0], lane, (uint32_t)(n - n_tiles * kTile));
+                                            accumulate, 1.0f, 0.0f, lds[0], lane, (uint32_t)(n - n_tiles * kTile));
         return;
     }
     const uint64_t tile = chunk_of<1, kAccBlock>(blockIdx.x, w, 0, xs);
     if (tile >= n_tiles) return;
     acc_tile<K, ALIGNED, MIX, false>(acc + tile * kTile, pl, k_payloads, tile * (kTile / 16), t, th, accumulate,
-                                     false, 1.0f, lds[w], lane);
+                                     1.0f, 0.0f, lds[w], lane);
 }
 
 // ---------------------------------------------------------------- matrix (n, k) kernels
@@ -840,16 +845,20 @@ struct QuantSegments {
     int count;
 };
 
-// Largest s with first[s] <= q (q < first[count]).
-__device__ __forceinline__ int find_segment(const uint32_t* first, int count, uint32_t q)
+// Largest s with first[s] <= q, for q < first[count]; the host fills first[count..96] with the total,
+// so the answer is the number of entries first[1..96) that are <= q.  Counted in two rounds of
+// independent scalar loads (7 pivots 12 entries apart, then the 11 entries behind the pivot) instead
+// of the 7 dependent loads of a binary search: a wave starts its memory traffic that much earlier.
+static_assert(kMaxSegments == 8 * 12, "find_segment splits the table into 8 blocks of 12");
+__device__ __forceinline__ int find_segment(const uint32_t* first, uint32_t q)
 {
-    int lo = 0, hi = count;  // invariant: first[lo] <= q < first[hi]
-    while (hi - lo > 1) {
-        const int mid = (lo + hi) >> 1;
-        if (first[mid] <= q) lo = mid;
-        else hi = mid;
-    }
-    return lo;
+    int block = 0;
+#pragma unroll
+    for (int p = 1; p < 8; ++p) block += first[12 * p] <= q ? 1 : 0;
+    int s = 12 * block;
+#pragma unroll
+    for (int j = 1; j < 12; ++j) s += first[12 * block + j] <= q ? 1 : 0;
+    return s;
 }
 
 template <bool ALIGNED, bool ADD, bool NT>
@@ -860,7 +869,7 @@ __global__ __launch_bounds__(256) void quant_multi_kernel(QuantSegments seg, uin
     const uint64_t q64 = chunk_of<1, 256>(blockIdx.x, w, 0, xs);
     if (q64 >= seg.first[seg.count]) return;
     const uint32_t q = (uint32_t)q64;
-    const int sidx = find_segment(seg.first, seg.count, q);
+    const int sidx = find_segment(seg.first, q);
     const float* g = seg.g[sidx];
     float* r = seg.r[sidx];
     uint32_t* c = seg.c[sidx];
@@ -911,26 +920,25 @@ struct AccSegments {
 template <int K, bool ALIGNED, bool MIX>
 __global__ __launch_bounds__(kAccBlock) void acc_multi_kernel(AccSegments seg, PayloadPtrs pl, int k_payloads,
                                                               uint32_t xs, float t, float th, int accumulate,
-                                                              float divisor)
+                                                              float divisor, float recip)
 {
-    const bool divide = divisor != 1.0f;
     __shared__ __attribute__((aligned(16))) float lds[kAccBlock / kWave][kAccLdsPerWave];
     const int lane = threadIdx.x & (kWave - 1);
     const uint32_t w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint64_t q64 = chunk_of<1, kAccBlock>(blockIdx.x, w, 0, xs);
     if (q64 >= seg.first[seg.count]) return;
     const uint32_t q = (uint32_t)q64;
-    const int sidx = find_segment(seg.first, seg.count, q);
+    const int sidx = find_segment(seg.first, q);
     const uint64_t n = seg.n[sidx];
     const uint64_t e0 = (uint64_t)(q - seg.first[sidx]) * kTile;
     if (e0 + kTile > n) {
         // last, shorter tile of the vector
         acc_tile<K, ALIGNED, MIX, true>(seg.acc[sidx] + e0, pl, k_payloads, seg.word_offset[sidx] + (e0 >> 4), t,
-                                        th, accumulate, divide, divisor, lds[w], lane, (uint32_t)(n - e0));
+                                        th, accumulate, divisor, recip, lds[w], lane, (uint32_t)(n - e0));
         return;
     }
     acc_tile<K, ALIGNED, MIX, false>(seg.acc[sidx] + e0, pl, k_payloads, seg.word_offset[sidx] + (e0 >> 4), t, th,
-                                     accumulate, divide, divisor, lds[w], lane);
+                                     accumulate, divisor, recip, lds[w], lane);
 }
 
 // ---------------------------------------------------------------- copy (measurement aid)
@@ -1128,6 +1136,16 @@ inline bool mix_ok(float t)
     return (b >> 31) == 0 && ex != 0xFFu && (ex >= 2 || b == 0);
 }
 
+// 1 / d when d is a power of two (other than 1) whose reciprocal is a normal number: then x * (1/d)
+// and x / d are the same real number and round to the same bits.  Else 0.
+inline float exact_reciprocal(float d)
+{
+    const uint32_t b = __builtin_bit_cast(uint32_t, d);
+    const uint32_t ex = (b >> 23) & 0xFFu;
+    if ((b & 0x007FFFFFu) != 0 || ex < 1 || ex > 253 || d == 1.0f) return 0.0f;
+    return __builtin_bit_cast(float, (b & 0x80000000u) | ((254u - ex) << 23));
+}
+
 // Instantiates BODY(K, AL, MIX) for the payload count k: K = k up to 8 (unrolled), else K = 0 (the
 // runtime-count form); the plain (non-MIX) form only exists with K = 0.
 #define NKLQ_ACC_DISPATCH(BODY, k, al, mix)                                          \
@@ -1312,9 +1330,10 @@ int launch_acc_multi(const AccSegments& seg, const PayloadPtrs& pl, int k, bool 
     const bool mix = mix_ok(t);
     const float th = -0.5f * t;
     const uint32_t pad = seg.first[seg.count] >= kAccThrottleTiles ? kAccThrottleLdsBytes : 0u;
+    const float recip = exact_reciprocal(divisor);
 #define NKLQ_AM(K, AL, MIX)                                                                           \
     launch_kernel((acc_multi_kernel<K, AL, MIX>), dim3(blocks), dim3(kAccBlock), pad, s, seg, pl, k, xs, \
-                       t, th, accumulate, divisor)
+                       t, th, accumulate, divisor, recip)
     NKLQ_ACC_DISPATCH(NKLQ_AM, k, al, mix);
 #undef NKLQ_AM
     return launch_status();

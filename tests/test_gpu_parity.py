@@ -355,6 +355,28 @@ def test_many_vectors_in_one_launch(knobs):
         assert_bits_equal(accs[i].cpu().numpy(), want, f"vector {i} n={n} divided")
 
 
+@pytest.mark.parametrize("divisor", [2.0, 8.0, 64.0, 0.25, -4.0, 2.0 ** 100, 2.0 ** -100, 2.0 ** 126, 2.0 ** -126,
+                                     2.0 ** 127, 2.0 ** -127, 3.0, 1.0000001, float("inf")])
+@pytest.mark.parametrize("thrd", [1e-3, 3e-38, 1e38])
+def test_division_folded_into_the_sum(divisor, thrd):
+    """The `/ kn` after the sum is a true IEEE division.  For a divisor that is a power of two the
+    kernel multiplies by the exact reciprocal instead, which must give the same bits everywhere:
+    quotients that are denormal, that underflow to zero, that overflow, and divisors whose
+    reciprocal is not a normal number (those, like every other divisor, are divided)."""
+    rng = np.random.default_rng(77)
+    n, K = 5000 + 11, 5
+    msgs = rng.integers(0, 2 ** 32, size=(K, (n + 15) // 16), dtype=np.uint64).astype(np.uint32)
+    base = (rng.standard_normal(n) * thrd * 2).astype(np.float32)
+    base[:4] = [0.0, -0.0, np.float32(thrd), -np.float32(thrd)]
+    for acc0 in (False, True):
+        acc = dev(base.copy())
+        q.cu_fn_dequantize_accumulate_multi_e([acc], [0], dev(msgs), thrd, accumulate=acc0, divisor=divisor)
+        with np.errstate(all="ignore"):
+            want = (oracle.c.dequant_accumulate(list(msgs), n, thrd, acc=base if acc0 else None)
+                    / np.float32(divisor)).astype(np.float32)
+        assert_bits_equal(acc.cpu().numpy(), want, f"divisor={divisor} thrd={thrd} accumulate={acc0}")
+
+
 def test_two_host_threads_on_two_streams():
     """The library keeps no per-call state: two host threads driving two streams at once get the
     same bits as one after the other."""
