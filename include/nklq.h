@@ -121,9 +121,9 @@ int nklq_dequant_accumulate_f32(float* acc, const uint32_t* const* payloads, int
  *
  * nklq_dequant_accumulate_multi_f32: for every i the fixed-order sum of nklq_dequant_accumulate_f32
  * into acc[i], where vector i's code words start at word_offset[i] inside each of the
- * k_payloads payload buffers payload_base[p] (one contiguous message per peer).  The sum is
- * divided by `divisor` (IEEE division) before it is stored unless divisor == 1: the `/ kn` that
- * follows the all-reduce at necklace/frmwrk/pytorch/ptprms.py:294.
+ * k_payloads payload buffers payload_base[p] (one contiguous message per peer).  Unless
+ * divisor == 1 the sum is divided by `divisor` before it is stored (the correctly rounded IEEE
+ * quotient): the `/ kn` that follows the all-reduce at necklace/frmwrk/pytorch/ptprms.py:294.
  */
 int nklq_quantize_multi_f32(int count, const float* const* g, float* const* r, uint32_t* const* c,
                             const uint64_t* n, float thrd, int add_residual, void* stream);

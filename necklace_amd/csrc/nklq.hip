@@ -832,7 +832,7 @@ __global__ __launch_bounds__(kBandsBlock) void deq_bands_kernel(
 // A model's gradients are many separate vectors (161 for ResNet-50, most of them small); one
 // launch per vector costs more in launch latency than the data takes to stream.  These kernels
 // take a table of up to kMaxSegments (96) vectors in their arguments and treat the chunks (or tiles)
-// of all of them as one index space; a wave finds its vector by binary search in the table.
+// of all of them as one index space; a wave finds its vector in the table (find_segment).
 
 constexpr int kMaxSegments = 96;  // 96 x 36 B of table stays under the 4 KiB kernel-argument limit
 
@@ -890,22 +890,35 @@ __global__ __launch_bounds__(256) void quant_multi_kernel(QuantSegments seg, uin
         const uint32_t word = quad_or(b << (8 * (lane & 3)));
         if ((lane & 3) == 0) c[(e0 >> 4) + (lane >> 2)] = word;
     } else {
-        // last, partial chunk of the vector: one element per lane, 4 rounds, all lanes reach row_or
-#pragma unroll
-        for (int first = 0; first < kChunk; first += kWave) {
-            const uint64_t e = e0 + (uint64_t)(first + lane);
-            const bool live = e < n;
-            uint32_t code = 0;
-            if (live) {
-                float a = g[e];
-                if constexpr (ADD) a = a + r[e];
+        // last, shorter chunk of the vector (rem = 1..255 elements): the same pass with the lanes past
+        // the end idle and the quad the end cuts going element by element; codes past the end are 0
+        const uint32_t rem = (uint32_t)(n - e0);
+        const uint32_t le = (uint32_t)lane * 4;
+        const float* gp = g + e0 + le;
+        float* rp = r + e0 + le;
+        uint32_t b = 0;
+        if (le + 4 <= rem) {
+            f32x4 v = ld4<ALIGNED, NT>(gp);
+            if constexpr (ADD) v = v + ld4<ALIGNED, NT>(rp);
+            float o0, o1, o2, o3;
+            b = quant_one(v.x, t, o0);
+            b |= quant_one(v.y, t, o1) << 2;
+            b |= quant_one(v.z, t, o2) << 4;
+            b |= quant_one(v.w, t, o3) << 6;
+            f32x4 o;
+            o.x = o0; o.y = o1; o.z = o2; o.w = o3;
+            st4<ALIGNED, NT>(rp, o);
+        } else if (le < rem) {
+            for (uint32_t i = 0; i < rem - le; ++i) {
+                float a = gp[i];
+                if constexpr (ADD) a = a + rp[i];
                 float res;
-                code = quant_one(a, t, res);
-                r[e] = res;
+                b |= quant_one(a, t, res) << (2 * i);
+                rp[i] = res;
             }
-            const uint32_t word = row_or(code << (2 * (lane & 15)));
-            if (live && (lane & 15) == 0) c[e >> 4] = word;
         }
+        const uint32_t word = quad_or(b << (8 * (lane & 3)));
+        if ((lane & 3) == 0 && le < rem) c[(e0 >> 4) + (lane >> 2)] = word;
     }
 }
 
