@@ -168,6 +168,23 @@ def test_config5_hbm_sizing_chunked_error_feedback():
             assert torch.equal(r_whole.view(torch.int32), r.view(torch.int32))
             del r_whole, c_whole
     assert int((c != 0).sum()) > 0
+    # the receive side at the same size, one launch each (element indices beyond 2^31): the decode
+    # of all 175,000,000 words and the sum of two payloads, into the gradient's buffer; first,
+    # middle and last chunk against the oracle
+    del r
+    c2 = c.clone()
+    c2[::3] = 0
+    q.cu_fn_matrix_dequantize_e(g, c, None, thrd)
+    for lo in (starts[0], starts[8], starts[-1]):
+        hi = min(n, lo + chunk)
+        want = oracle.c.dequantize(host_words(c[lo // 16:(hi + 15) // 16]), hi - lo, thrd)
+        assert torch.equal(g[lo:hi].view(torch.int32), dev(want).view(torch.int32)), f"decode of chunk at {lo}"
+    q.cu_fn_dequantize_accumulate_e(g, [c, c2], thrd)
+    for lo in (starts[0], starts[8], starts[-1]):
+        hi = min(n, lo + chunk)
+        pl = [host_words(x[lo // 16:(hi + 15) // 16]) for x in (c, c2)]
+        want = oracle.c.dequant_accumulate(pl, hi - lo, thrd)
+        assert torch.equal(g[lo:hi].view(torch.int32), dev(want).view(torch.int32)), f"sum of chunk at {lo}"
 
 
 @pytest.mark.parametrize("n,k", [(4099, 8191), (1_000_003, 17), (100_003, 384), (50_001, 385), (2_000_001, 3)])
