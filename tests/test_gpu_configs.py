@@ -208,6 +208,45 @@ def test_large_matrices_every_kernel_regime_against_the_oracle(n, k):
     assert_bits_equal(R.cpu().numpy(), oracle.c.dequantize(want_c, n, thrd), f"{n}x{k} decode")
 
 
+@pytest.mark.parametrize("n,k", [(46_349, 46_341), (268_435_461, 9)])
+def test_matrix_forms_beyond_2_31_elements(n, k):
+    """Matrices of more than 2^31 elements (8.6 and 9.7 GB per array) through the row kernels and
+    the band kernels in one launch: slabs of whole word rows at the start, either side of element
+    2^31, and at the ragged end are checked against the oracle (a slab of rows 16a..16b of a
+    row-major matrix is a matrix of its own, with the word rows a..b)."""
+    thrd, m = 2e-3, (n + 15) // 16
+    assert n * k > 2 ** 31
+    A = torch.empty(n, k, device="cuda")
+    R = torch.empty(n, k, device="cuda")
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(n % 1000 + k)
+    rows_per_piece = max(16, (1 << 26) // k // 16 * 16)
+    for lo in range(0, n, rows_per_piece):
+        hi = min(n, lo + rows_per_piece)
+        torch.randn(hi - lo, k, device="cuda", generator=gen, out=A[lo:hi])
+        torch.randn(hi - lo, k, device="cuda", generator=gen, out=R[lo:hi])
+    A.mul_(1e-3)
+    R.mul_(1e-3)
+    C = torch.full((m, k), -1, dtype=torch.int32, device="cuda")
+    slab = max(1, (1 << 22) // (16 * k))                      # word rows per slab: about 4 M elements
+    mid = (2 ** 31 // k) // 16                                # the word row that holds element 2^31
+    slabs = [(0, slab), (max(0, mid - slab // 2), min(m, mid + slab)), (m - slab, m)]
+    before = [(A[16 * a:min(n, 16 * b)].cpu().numpy(), R[16 * a:min(n, 16 * b)].cpu().numpy()) for a, b in slabs]
+    q.cu_fn_matrix_quantize_e(A, C, R, thrd, add_residual=True)
+    wants = []
+    for (a, b), (a_host, r_host) in zip(slabs, before):
+        want_c, want_r = oracle.c.quantize(a_host, thrd, R_in=r_host)
+        assert_words_equal(C[a:b].cpu().numpy().view(np.uint32), want_c, f"{n}x{k} codes of word rows {a}..{b}")
+        assert_bits_equal(R[16 * a:min(n, 16 * b)].cpu().numpy(), want_r, f"{n}x{k} residual of word rows {a}..{b}")
+        wants.append(want_c)
+    assert int((C == -1).sum()) == 0                          # every word was written: no code is ever 11
+    q.cu_fn_matrix_dequantize_e(A, C, None, thrd)
+    for (a, b), want_c in zip(slabs, wants):
+        rows = min(n, 16 * b) - 16 * a
+        assert_bits_equal(A[16 * a:16 * a + rows].cpu().numpy(), oracle.c.dequantize(want_c, rows, thrd),
+                          f"{n}x{k} decode of word rows {a}..{b}")
+
+
 @pytest.mark.parametrize("og,orr,oo", [(1, 1, 1), (0, 3, 31), (4, 4, 8), (16, 0, 16), (0, 16, 5)])
 def test_large_flat_views_off_cache_lines(og, orr, oo):
     """20 M elements cut out of larger buffers at element offsets: the residual (and the decode
