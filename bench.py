@@ -16,7 +16,9 @@ fp32 elements, inputs resident in HBM.  Prints one JSON line:
   extras       decode (elements/s), 8-payload fixed-order sum, plain copy, the other four
                synthetic workloads (config1, config2, config3, config5: kernel time, GB/s of
                algorithmic bytes, fraction of the HBM peak), wall time per call of the
-               reference-named wrapper at small sizes
+               reference-named wrapper at small sizes, the matrix form on seven shapes (wide,
+               rows off cache lines, a few columns), a ResNet-50-shaped list of 161 gradient
+               tensors through the trainer-side buffers
 
 The CPU checker is used for the cpu_baseline leg only, never for the GPU path.
 """
@@ -48,9 +50,9 @@ def parse():
                     help="elements per launch (multiple of 16); 0 = the whole gradient in one launch. "
                          "The HBM-sizing workload is --elems 2800000000 --chunk 268435456")
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="CPU-baseline time budget; 0 skips it")
-    ap.add_argument("--legs", default="deq,acc,configs,wrapper,copy,cpu",
-                    help="extra legs after the timed quantize steps: deq, acc, configs, wrapper, copy, cpu, "
-                         "and (off by default) matrix, multi, accsweep (comma list, '' = none)")
+    ap.add_argument("--legs", default="deq,acc,configs,wrapper,matrix,multi,copy,cpu",
+                    help="extra legs after the timed quantize steps: deq, acc, configs, wrapper, matrix, multi, "
+                         "copy, cpu, and (off by default) accsweep (comma list, '' = none)")
     return ap.parse_args()
 
 
