@@ -16,7 +16,7 @@ fp32 elements, inputs resident in HBM.  Prints one JSON line:
   extras       decode (elements/s), 8-payload fixed-order sum, plain copy, the other four
                synthetic workloads (config1, config2, config3, config5: kernel time, GB/s of
                algorithmic bytes, fraction of the HBM peak), wall time per call of the
-               reference-named wrapper at small sizes, the matrix form on seven shapes (wide,
+               reference-named wrapper at small sizes, the matrix form on eight shapes (wide,
                rows off cache lines, a few columns), a ResNet-50-shaped list of 161 gradient
                tensors through the trainer-side buffers
 
@@ -606,8 +606,8 @@ def main():
         # the reference's own layout: (n, k) matrix, codes packed down the columns; wide and narrow,
         # rows on and off 128-byte lines
         res["matrix"] = {}
-        for rows, cols in ((8192, 8192), (8191, 8191), (16384, 16383), (100000, 1000), (20_000_000, 3),
-                           (4_000_000, 17), (1_000_000, 65)):
+        for rows, cols in ((8192, 8192), (8191, 8191), (16384, 16383), (100000, 1000), (150_000, 401),
+                           (20_000_000, 3), (4_000_000, 17), (1_000_000, 65)):
             tot = rows * cols
             A = g[:tot] if tot <= n else torch.randn(tot, device="cuda", generator=gen) * 1e-3
             R = torch.zeros(tot, device="cuda")

@@ -682,6 +682,12 @@ __global__ __launch_bounds__(kRowsBlock) void deq_2d_rows_kernel(
 // LDS; after a barrier the words are stored, contiguous.
 constexpr int kBandsBlock = 256;
 constexpr uint64_t kBandsMaxColumns = 384;  // LDS words per workgroup; wider matrices take the row tiles (measured crossover: 300-500 columns)
+// The decode also takes bands for up to 800 columns when most rows start off a 16-byte boundary
+// (an odd k, or a base off one): the row tiles then cut a quad at both ends of nearly every row
+// and measured 0.45-0.60 of the HBM peak at 385..799 columns against 0.60-0.67 here; with whole
+// quads in every row, or every other row (k = 2 mod 4), the row tiles are as fast or faster
+// (0.62-0.93) and keep those shapes.
+constexpr uint64_t kBandsMaxColumnsDecode = 800;
 constexpr uint64_t kBandsRangeQuant = 2048;   // elements per workgroup when bands are short: quantize
 constexpr uint64_t kBandsRangeDecode = 4096;  // and decode (measured)
 
@@ -791,7 +797,7 @@ __global__ __launch_bounds__(kBandsBlock) void deq_bands_kernel(
     float* out, const uint32_t* __restrict__ c, uint64_t n, uint32_t k, uint32_t bands_per_wg, uint32_t inv,
     float t)
 {
-    __shared__ uint32_t words[kBandsMaxColumns];
+    __shared__ uint32_t words[kBandsMaxColumnsDecode];
     const uint64_t m = (n + 15) / 16;
     const uint64_t x0 = (uint64_t)blockIdx.x * bands_per_wg;  // (runs per XCD measured slower for the decode)
     const uint64_t x1 = (x0 + bands_per_wg < m) ? x0 + bands_per_wg : m;
@@ -1517,7 +1523,8 @@ int nklq_dequantize_f32(float* out, const uint32_t* c, uint64_t n_rows, uint64_t
         return dispatch_deq_flat(out, c, total, thrd, s);
     }
     const uint64_t m = n_rows / 16 + (n_rows % 16 ? 1 : 0);
-    if (n_cols <= kBandsMaxColumns) {
+    if (n_cols <= kBandsMaxColumns ||
+        (n_cols <= kBandsMaxColumnsDecode && (n_cols % 2 != 0 || !aligned16(out)))) {
         uint32_t per;
         const uint32_t grid = bands_grid(n_rows, n_cols, kBandsRangeDecode, false, &per);
         if (grid == 0) return NKLQ_ERANGE;

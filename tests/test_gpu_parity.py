@@ -139,7 +139,8 @@ def test_matrix_layout(n, k):
 
 
 @pytest.mark.parametrize("n,k", [(5000, 3), (2003, 17), (700, 255), (100, 257), (130, 511), (40, 1023), (40, 1024),
-                                 (40, 1025), (33, 1030), (50, 4099), (20, 8191), (129, 2048), (16, 1000)])
+                                 (40, 1025), (33, 1030), (50, 4099), (20, 8191), (129, 2048), (16, 1000),
+                                 (300, 384), (300, 385), (70, 513), (90, 666), (49, 799), (64, 800), (64, 801)])
 @pytest.mark.parametrize("og,orr,oc", [(0, 0, 0), (1, 1, 1), (3, 2, 0), (0, 1, 3)])
 def test_matrix_forms_inside_larger_buffers(n, k, og, orr, oc):
     """Every column regime (bands of a few columns, one band per workgroup, row tiles; k a multiple
