@@ -497,20 +497,48 @@ def _reduce_params_form(nc, kn, root, params, cfg):
     _reduce_small(small, kn, _small_fn(nc, cfg, root), average)
 
 
+def _bucket_places(owners, buckets):
+    """{id of parameter: (bucket, offset, numel)} for a bucketing of the parameters' gradients."""
+    places, it = {}, iter(owners)
+    for bi, bucket in enumerate(buckets):
+        pos = 0
+        for g in bucket:
+            places[next(it)] = (bi, pos, g.numel())
+            pos += g.numel()
+    return places
+
+
 def _reduce_buckets_form(nc, kn, root, params, cfg):
-    grads = [p.grad.data for p in params if p.grad is not None]
+    live = [p for p in params if p.grad is not None]
+    grads = [p.grad.data for p in live]
     if not grads:
         return
     buckets = _take_buckets(grads, int(cfg.get("bucket_bytes", NCCL_REDUCE_BUCKET_BYTES)))
     sizes = [sum(g.numel() for g in b) for b in buckets]
     sig = ("buckets", tuple(tuple(g.numel() for g in b) for b in buckets), kn)
-    if cfg.get("_signature") != sig:
+    places = _bucket_places([id(p) for p in live], buckets)
+    if cfg.get("_signature") != sig or cfg.get("_places") != places:
+        old_gc, old_places = cfg.get("compressor"), cfg.get("_places")
+        was_buckets = cfg.get("_signature", ("",))[0] == "buckets"
         sub = dict(cfg)
         sub["grad_size_threshold"] = 1  # a bucket is always packed
         built = init_grad_comp_cfg(sizes, kn, sub, device=grads[0].device, rank=cfg.get("rank", 0))
+        if was_buckets and old_places:
+            # the set of gradients changed: what a parameter is still owed moves to its new place;
+            # a parameter that sits this step out has its residual set aside until it comes back
+            parked = cfg.setdefault("_parked", {})
+            for pid, was in old_places.items():
+                if pid not in places:
+                    parked[pid] = old_gc.grd_resi[was[0]][was[1]:was[1] + was[2]].clone()
+            for pid, (bi, pos, n) in places.items():
+                was = old_places.get(pid)
+                if was is not None and was[2] == n:
+                    built["grd_resi"][bi][pos:pos + n].copy_(old_gc.grd_resi[was[0]][was[1]:was[1] + n])
+                elif was is None and pid in parked and parked[pid].numel() == n:
+                    built["grd_resi"][bi][pos:pos + n].copy_(parked.pop(pid))
         for key in ("grd_resi", "grd_recv", "grd_comp", "grd_cmps", "compressor"):
             cfg[key] = built[key]
-        cfg["_signature"] = sig
+        cfg["_signature"], cfg["_places"] = sig, places
         cfg["_flat"] = [torch.empty(n, dtype=torch.float32, device=grads[0].device) for n in sizes]
     gc, flats = cfg["compressor"], cfg["_flat"]
     for flat, bucket in zip(flats, buckets):  # grads_batch_coalesced, ptprms.py:262

@@ -329,6 +329,49 @@ def test_bucket_form_packs_flattened_buckets_like_nccl_allreduce_by_buckets():
     assert all(c[0] == "gather" for c in nc.calls)  # nothing stays fp32 in this form
 
 
+def test_bucket_form_keeps_what_is_owed_when_the_set_of_gradients_changes():
+    """Bucket form, three steps; at step 2 one parameter has no gradient, at step 3 it is back: the
+    buckets are laid out anew both times and every parameter's residual moves to its new place
+    (the one that sat out keeps what it was owed at step 1... which a fresh layout would drop)."""
+    model, opt, x, y = _mlp_with_grads(seed=9)
+    params = list(model.parameters())
+    thrd, kn, limit = 1e-3, 2, 1 << 19
+    cfg = {"grad_comp_threshold": thrd, "form": "buckets", "bucket_bytes": limit}
+    nc = TwoWorkersWithEqualData()
+    owed = {i: np.zeros(p.numel(), np.float32) for i, p in enumerate(params)}
+    absent = 2  # the second layer's weight
+    for step in range(3):
+        if step:
+            opt.zero_grad(set_to_none=False)
+            torch.nn.functional.cross_entropy(model(x), y).backward()
+        if step == 1:
+            params[absent].grad = None
+        live = [i for i, p in enumerate(params) if p.grad is not None]
+        grads = {i: params[i].grad.detach().cpu().numpy().reshape(-1).copy() for i in live}
+        ptcomp.opt_grads_do_nccl_allreduce(nc, kn, opt, None, grad_comp_cfg=cfg)
+        torch.cuda.synchronize()
+        buckets, cur, size = [], [], 0
+        for i in live:
+            if cur and size + 4 * grads[i].size > limit:
+                buckets.append(cur)
+                cur, size = [], 0
+            cur.append(i)
+            size += 4 * grads[i].size
+        buckets.append(cur)
+        for b in buckets:
+            flat = np.concatenate([grads[i] for i in b])
+            c, r = oracle.c.quantize(flat, thrd, R_in=np.concatenate([owed[i] for i in b]))
+            want = (oracle.c.dequant_accumulate([c, c], flat.size, thrd) / np.float32(kn)).astype(np.float32)
+            pos = 0
+            for i in b:
+                n = grads[i].size
+                owed[i] = r[pos:pos + n].copy()
+                assert_bits_equal(params[i].grad.detach().cpu().numpy().reshape(-1), want[pos:pos + n],
+                                  f"step {step} parameter {i}")
+                pos += n
+    assert float(np.abs(owed[absent]).sum()) > 0
+
+
 def test_sgd_with_compressed_gradients_still_learns():
     """End to end on one worker: every step's gradients go through compress -> decompress (2 bits
     per element plus error feedback) before the optimizer sees them, and the model still fits."""
