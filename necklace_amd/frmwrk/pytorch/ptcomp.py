@@ -621,9 +621,17 @@ def opt_grads_do_nccl_reduce(nc, kn, root, opt, prm_revs=None, grad_comp_cfg=Non
 
 def opt_grads_fltn_do_nccl_reduce(nc, kn, root, d_arr_send, sz, grad_comp_cfg=None):
     """Compressed counterpart of ptprms.opt_grads_fltn_do_nccl_reduce (ptprms.py:396-401) on the
-    flat gradient buffer; see `opt_grads_fltn_do_compressed_reduce`.  Only `root` decodes."""
-    if grad_comp_cfg is None or "compressor" not in grad_comp_cfg:
-        raise ValueError("build grad_comp_cfg with init_flat_grad_comp_cfg first")
-    gc = grad_comp_cfg["compressor"]
+    flat gradient buffer; see `opt_grads_fltn_do_compressed_reduce`.  Only `root` decodes.  The
+    buffers are laid out on the first call (or by `init_flat_grad_comp_cfg` beforehand) and kept in
+    `grad_comp_cfg`."""
+    if grad_comp_cfg is None:
+        raise ValueError("grad_comp_cfg is required: this is the compressed path")
+    gc = grad_comp_cfg.get("compressor")
+    if gc is None or gc.kn != kn or list(gc.layout.numels) != [int(sz)]:
+        # first call (or another buffer length): lay the buffers out next to the flat gradient;
+        # a residual from before belongs to another layout and does not carry over
+        grad_comp_cfg.update(init_flat_grad_comp_cfg(sz, kn, grad_comp_cfg, device=d_arr_send.device,
+                                                     rank=grad_comp_cfg.get("rank", 0)))
+        gc = grad_comp_cfg["compressor"]
     opt_grads_fltn_do_compressed_reduce(kn, d_arr_send, sz, grad_comp_cfg, exchange=_exchange_of(nc),
                                         average=False, decode=gc.rank == root)

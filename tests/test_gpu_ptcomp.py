@@ -126,6 +126,34 @@ def test_flat_zero_style_buffer_reduce_in_place():
         assert_bits_equal(buf.cpu().numpy(), oracle.c.dequant_accumulate(pl, total, thrd), f"step {step}")
 
 
+def test_flat_buffer_drop_in_under_the_reference_name():
+    """ptprms.opt_grads_fltn_do_nccl_reduce(nc, kn, root, d_arr_send, sz, grad_comp_cfg=...)
+    (necklace/frmwrk/pytorch/ptprms.py:396-401) with nothing but the trainer's own dict: the
+    buffers are laid out on the first call; the root ends with the decoded sum (not averaged, as
+    the reference's reduce), the other worker keeps its gradient; two steps of error feedback."""
+    n, kn, thrd = 300_000 + 7, 2, 1e-3
+    rng = np.random.default_rng(8)
+    for rank, root in ((0, 0), (1, 0)):
+        cfg = {"grad_comp_threshold": thrd, "rank": rank}
+        nc = TwoWorkersWithEqualData(rank=rank)
+        resid = np.zeros(n, np.float32)
+        for step in range(2):
+            g = rng.normal(0, 1e-3, n + 5).astype(np.float32)
+            buf = dev(g)                                   # the flat buffer is longer than what is sent
+            assert ptcomp.opt_grads_fltn_do_nccl_reduce(nc, kn, root, buf, n, grad_comp_cfg=cfg) is None
+            torch.cuda.synchronize()
+            c, resid = oracle.c.quantize(g[:n], thrd, R_in=resid)
+            assert_bits_equal(cfg["compressor"].grd_resi[0].cpu().numpy(), resid, f"rank {rank} step {step}")
+            got = buf.cpu().numpy()
+            assert_bits_equal(got[n:], g[n:], "past sz")
+            if rank == root:
+                assert_bits_equal(got[:n], oracle.c.dequant_accumulate([c, c], n, thrd), f"root, step {step}")
+            else:
+                assert_bits_equal(got[:n], g[:n], f"not the root, step {step}")
+    with pytest.raises(ValueError):
+        ptcomp.opt_grads_fltn_do_nccl_reduce(None, 1, 0, dev(np.zeros(64, np.float32)), 64, grad_comp_cfg=None)
+
+
 def test_checkpoint_file_round_trip(tmp_path):
     n, thrd = 20_000, 1e-3
     cfg = ptcomp.init_flat_grad_comp_cfg(n, 1, {"grad_comp_threshold": thrd})
