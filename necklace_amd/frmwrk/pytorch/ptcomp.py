@@ -591,6 +591,16 @@ def grads_do_nccl_allreduce(nc, kn, model, prm_revs=None, grad_comp_cfg=None):
     _reduce_params(nc, kn, None, params, grad_comp_cfg)
 
 
+def grads_do_nccl(params, prm_recvs, nc, kn, grad_comp_cfg=None):
+    """The call the MXNet trainer makes, ``mxprms.grads_do_nccl(net.collect_params(), prm_recvs,
+    nc, kn, grad_comp_cfg=...)`` (necklace/trainer/tnopmx.py:334-337), with its argument order:
+    `params` is a sequence of parameters or a dict of them (the values are taken, in order), each
+    with a ``.grad``; `prm_recvs` (the fp32 receive buffers of the uncompressed path) is not needed
+    here.  Every gradient ends as the average over the `kn` workers.  Returns None."""
+    plist = list(params.values()) if hasattr(params, "values") else list(params)
+    _reduce_params(nc, kn, None, plist, grad_comp_cfg)
+
+
 def opt_one_grads_do_nccl_allreduce(nc, kn, opt, prm_revs=None, grad_comp_cfg=None):
     """Compressed counterpart of ptprms.opt_one_grads_do_nccl_allreduce
     (necklace/frmwrk/pytorch/ptprms.py:329-338): afterwards EVERY gradient of the optimizer holds

@@ -257,6 +257,13 @@ def test_model_form_gives_what_the_optimizer_form_gives():
     torch.cuda.synchronize()
     for pa, pb in zip(model_a.parameters(), model_b.parameters()):
         assert torch.equal(pa.grad, pb.grad)
+    # the MXNet trainer's call shape: a dict of parameters, the receive buffers, nc, kn
+    model_d, _, _, _ = _mlp_with_grads(seed=5)
+    assert ptcomp.grads_do_nccl(dict(model_d.named_parameters()), None, TwoWorkersWithEqualData(), kn,
+                                grad_comp_cfg=dict(cfg_a)) is None
+    torch.cuda.synchronize()
+    for pa, pd in zip(model_a.parameters(), model_d.parameters()):
+        assert torch.equal(pa.grad, pd.grad)
     # a frozen parameter is not part of the layout, its stale gradient is left alone
     model_c, _, _, _ = _mlp_with_grads(seed=5)
     first = next(model_c.parameters())
