@@ -52,7 +52,7 @@ def parse():
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="CPU-baseline time budget; 0 skips it")
     ap.add_argument("--legs", default="deq,acc,configs,wrapper,matrix,multi,copy,cpu",
                     help="extra legs after the timed quantize steps: deq, acc, configs, wrapper, matrix, multi, "
-                         "copy, cpu, and (off by default) accsweep (comma list, '' = none)")
+                         "copy, cpu, and (off by default) accsweep, geometry (comma list, '' = none)")
     return ap.parse_args()
 
 
@@ -477,7 +477,7 @@ def main():
     }
 
     legs = {x for x in args.legs.split(",") if x}
-    if legs & {"deq", "copy"}:
+    if legs & {"deq", "copy", "geometry"}:
         out = torch.empty(n, dtype=torch.float32, device="cuda")
     if "deq" in legs:
 
@@ -601,6 +601,47 @@ def main():
                 "us": round(ev / 20 * 1e3, 1), "GBps": round(gb, 1), "frac_hbm_peak": frac(gb),
                 "payload_MB": round(4 * wl * kp / 1e6)}
         del big, accl
+
+    if "geometry" in legs:
+        # the launch knobs of nklq_tune on the three flat kernels at gradient size: the shipped defaults
+        # against their neighbours (results never depend on them, only the time does)
+        import ctypes as ct
+        default = [_lib.tune(i) for i in range(_lib.N_TUNE)]
+        wl = _lib.packed_words(n)
+        pay = torch.randint(-2 ** 31, 2 ** 31 - 1, (K_PAYLOADS, wl), dtype=torch.int32, device="cuda", generator=gen)
+        ptrg = (ct.c_void_p * K_PAYLOADS)(*[pay[p].data_ptr() for p in range(K_PAYLOADS)])
+        kernels = {
+            "quantize": (lambda: _lib.check(L.nklq_quantize_f32(gp, rp, rp, cp, n, 1, THRD, 1, stream)), BYTES_QUANT),
+            "decode": (lambda: _lib.check(L.nklq_dequantize_f32(out.data_ptr(), cp, n, 1, THRD, stream)), BYTES_DEQUANT),
+            "sum8": (lambda: _lib.check(L.nklq_dequant_accumulate_f32(out.data_ptr(), ptrg, K_PAYLOADS, n, THRD, 0, stream)),
+                     0.25 * K_PAYLOADS + 4),
+        }
+        sweeps = {   # kernel -> [(label, {knob: value})]
+            "quantize": [(f"interleave 2^{x}", {_lib.TUNE_XCD_INTERLEAVE_LOG2: x}) for x in range(7)]
+                        + [(f"{u} chunks per wave", {_lib.TUNE_CHUNKS_PER_WAVE: u}) for u in (2, 4)]
+                        + [(f"workgroup {b}", {_lib.TUNE_WORKGROUP_SIZE: b}) for b in (64, 128, 512, 1024)]
+                        + [("cached loads and stores", {_lib.TUNE_NONTEMPORAL: 0})],
+            "decode": [(f"interleave 2^{x}", {_lib.TUNE_XCD_INTERLEAVE_LOG2_DECODE: x}) for x in range(7)]
+                      + [("cached stores", {_lib.TUNE_NONTEMPORAL: 0})],
+            "sum8": [(f"interleave 2^{x}", {_lib.TUNE_XCD_INTERLEAVE_LOG2_ACCUMULATE: x}) for x in range(7)],
+        }
+        res["launch_geometry"] = {"defaults": default}
+        for name, (fn, bpe) in kernels.items():
+            rows_ = {}
+            for label, knobs in [("defaults", {})] + sweeps[name]:
+                for i, v in enumerate(default):
+                    _lib.tune(i, v)
+                for kk, v in knobs.items():
+                    _lib.tune(kk, v)
+                for _ in range(5):
+                    fn()
+                _, ev = time_region(torch, fn, 10)
+                gb = bpe * n / (ev / 10 * 1e-3) / 1e9
+                rows_[label] = {"us": round(ev / 10 * 1e3, 1), "frac_hbm_peak": frac(gb)}
+            res["launch_geometry"][name] = rows_
+        for i, v in enumerate(default):
+            _lib.tune(i, v)
+        del pay
 
     if "matrix" in legs:
         # the reference's own layout: (n, k) matrix, codes packed down the columns; wide and narrow,
