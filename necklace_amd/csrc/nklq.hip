@@ -813,22 +813,35 @@ __global__ __launch_bounds__(kBandsBlock) void deq_bands_kernel(
     for (int32_t li = -(int32_t)a + 4 * (int32_t)threadIdx.x; li < (int32_t)len; li += 4 * kBandsBlock) {
         uint32_t row, col;
         band_row_col((uint32_t)(li < 0 ? 0 : li), k, inv, &row, &col);
-        float o[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            if (li + j >= 0 && li + j < (int32_t)len) {
-                o[j] = deq_code((words[(row >> 4) * k + col] >> (2 * (row & 15u))) & 3u, t);
-                if (++col == k) { col = 0; ++row; }
-            }
-        }
         if (li >= 0 && li + 4 <= (int32_t)len) {
+            // a whole quad (all but the first and last of a range): no bounds to check
             f32x4 vo;
-            vo.x = o[0]; vo.y = o[1]; vo.z = o[2]; vo.w = o[3];
+            if (col + 4 <= k) {
+                // inside one row, the usual case: one word address and one bit position for all four
+                const uint32_t* wq = &words[(row >> 4) * k + col];
+                const uint32_t sh = 2 * (row & 15u);
+                vo.x = deq_code((wq[0] >> sh) & 3u, t);
+                vo.y = deq_code((wq[1] >> sh) & 3u, t);
+                vo.z = deq_code((wq[2] >> sh) & 3u, t);
+                vo.w = deq_code((wq[3] >> sh) & 3u, t);
+            } else {
+                float o[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    o[j] = deq_code((words[(row >> 4) * k + col] >> (2 * (row & 15u))) & 3u, t);
+                    if (++col == k) { col = 0; ++row; }
+                }
+                vo.x = o[0]; vo.y = o[1]; vo.z = o[2]; vo.w = o[3];
+            }
             st4<true, NT>(oq + li, vo);
         } else {
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-                if (li + j >= 0 && li + j < (int32_t)len) oq[li + j] = o[j];
+            for (int j = 0; j < 4; ++j) {
+                if (li + j >= 0 && li + j < (int32_t)len) {
+                    oq[li + j] = deq_code((words[(row >> 4) * k + col] >> (2 * (row & 15u))) & 3u, t);
+                    if (++col == k) { col = 0; ++row; }
+                }
+            }
         }
     }
 }
