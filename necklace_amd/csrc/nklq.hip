@@ -277,8 +277,9 @@ __global__ __launch_bounds__(256) void quant_flat_offline_kernel(
 // out[j] = decode(c)[j]  (the reference dequantize, flat).  The 4 lanes of a quad read the
 // same code word (one 64 B request per wave) and each takes its byte.  Code words are read
 // with ordinary (cached) loads: two chunks share a 128 B line, and non-temporal loads of half
-// lines measure 20-35 % slower here.
-template <int U, int BLOCK, bool ALIGNED, bool NT>
+// lines measure 20-35 % slower here.  The target starts on a 128-byte line (any other start takes
+// deq_flat_shift_kernel), so every store is a whole aligned 16 bytes.
+template <int U, int BLOCK, bool NT>
 __global__ __launch_bounds__(BLOCK) void deq_flat_kernel(
     float* out, const uint32_t* __restrict__ c, uint64_t n, uint64_t n_chunks, uint32_t has_tail,
     uint32_t xs, float t)
@@ -300,7 +301,7 @@ __global__ __launch_bounds__(BLOCK) void deq_flat_kernel(
         const uint64_t ch = chunk_of<U, BLOCK>(blockIdx.x, w, j, xs);
         if (ch >= n_chunks) continue;
         const uint32_t word = c[ch * kWordsPerChunk + (lane >> 2)];
-        st4<ALIGNED, NT>(out + ch * kChunk + lane * 4, deq_byte((word >> sh) & 0xFFu, t));
+        st4<true, NT>(out + ch * kChunk + lane * 4, deq_byte((word >> sh) & 0xFFu, t));
     }
 }
 
@@ -1055,17 +1056,20 @@ inline int launch_status() { return t_launch_status; }
 
 // ---- overlap checks
 //
-// Byte ranges of the buffers of a call.  An output may coincide EXACTLY with an input (the in-place
-// forms: r_out == r_in, r_out == g); any other overlap that involves an output is refused.
+// Byte ranges of the buffers of a call.  An output may coincide EXACTLY with an input that is named
+// as its in-place partner (r_out == r_in, r_out == g: each element is read and then written by the
+// same lane); any other overlap that involves an output is refused, also an exact coincidence with
+// an input that is not its partner (the code words on top of a one-row gradient, say).
 struct Span {
     uintptr_t lo, hi;
     bool out;
+    int tag;  // an output: its own id; an input: the id of the output it may coincide with, or -1
 };
 
-inline Span span_of(const void* p, uint64_t bytes, bool out)
+inline Span span_of(const void* p, uint64_t bytes, bool out, int tag = -1)
 {
     const uintptr_t lo = reinterpret_cast<uintptr_t>(p);
-    return Span{lo, lo + (uintptr_t)bytes, out};
+    return Span{lo, lo + (uintptr_t)bytes, out, tag};
 }
 
 bool spans_conflict(std::vector<Span>& v)
@@ -1077,11 +1081,13 @@ bool spans_conflict(std::vector<Span>& v)
     });
     uintptr_t end_out = 0, end_any = 0;  // furthest end among the outputs / all ranges seen so far
     uintptr_t out_lo = 0, out_hi = 0;    // the latest output
+    int out_tag = -1;
     for (size_t i = 0; i < v.size(); ++i) {
         if (v[i].lo == v[i].hi) continue;
-        // inputs identical to the output sorted just before them are that output's in-place partners
-        const bool partner = !v[i].out && out_hi != 0 && v[i].lo == out_lo && v[i].hi == out_hi;
-        if (v[i].out) { out_lo = v[i].lo; out_hi = v[i].hi; }
+        // inputs identical to the output sorted just before them, and named as its partner, are in place
+        const bool partner = !v[i].out && out_hi != 0 && v[i].lo == out_lo && v[i].hi == out_hi &&
+                             v[i].tag >= 0 && v[i].tag == out_tag;
+        if (v[i].out) { out_lo = v[i].lo; out_hi = v[i].hi; out_tag = v[i].tag; }
         if (!partner) {
             if (v[i].out ? v[i].lo < end_any : v[i].lo < end_out) return true;
         }
@@ -1146,16 +1152,12 @@ int launch_deq_flat(float* out, const uint32_t* c, uint64_t n, float t, hipStrea
 {
     const FlatGrid fg = flat_grid(n, U, BLOCK, tk.xcd_shift_decode);
     if (fg.blocks == 0) return NKLQ_ERANGE;
-    const bool al = aligned16(out);
-    const bool nt = tk.nontemporal != 0;
-#define NKLQ_DEQ(AL, NT)                                                                        \
-    launch_kernel((deq_flat_kernel<U, BLOCK, AL, NT>), dim3(fg.blocks), dim3(BLOCK), 0, s, out, \
-                       c, n, fg.n_chunks, fg.has_tail, fg.xs, t)
-    if (al && nt) NKLQ_DEQ(true, true);
-    else if (al) NKLQ_DEQ(true, false);
-    else if (nt) NKLQ_DEQ(false, true);
-    else NKLQ_DEQ(false, false);
-#undef NKLQ_DEQ
+    if (tk.nontemporal)
+        launch_kernel((deq_flat_kernel<U, BLOCK, true>), dim3(fg.blocks), dim3(BLOCK), 0, s, out, c, n,
+                      fg.n_chunks, fg.has_tail, fg.xs, t);
+    else
+        launch_kernel((deq_flat_kernel<U, BLOCK, false>), dim3(fg.blocks), dim3(BLOCK), 0, s, out, c, n,
+                      fg.n_chunks, fg.has_tail, fg.xs, t);
     return launch_status();
 }
 
@@ -1450,10 +1452,10 @@ int nklq_quantize_f32(const float* g, const float* r_in, float* r_out, uint32_t*
         return NKLQ_EALIGN;
     const bool add = add_residual != 0;
     {
-        std::vector<Span> spans = {span_of(r_out, 4 * total, true),
-                                   span_of(c, 4 * nklq_packed_words(n_rows, n_cols), true),
-                                   span_of(g, 4 * total, false)};
-        if (add) spans.push_back(span_of(r_in, 4 * total, false));
+        std::vector<Span> spans = {span_of(r_out, 4 * total, true, 0),
+                                   span_of(c, 4 * nklq_packed_words(n_rows, n_cols), true, 1),
+                                   span_of(g, 4 * total, false, 0)};
+        if (add) spans.push_back(span_of(r_in, 4 * total, false, 0));
         if (spans_conflict(spans)) return NKLQ_EALIAS;
     }
     snapshot_knobs();
@@ -1526,7 +1528,7 @@ int nklq_dequantize_f32(float* out, const uint32_t* c, uint64_t n_rows, uint64_t
     if (!out || !c) return NKLQ_ENULL;
     if (!aligned4(out) || !aligned4(c)) return NKLQ_EALIGN;
     {
-        std::vector<Span> spans = {span_of(out, 4 * total, true),
+        std::vector<Span> spans = {span_of(out, 4 * total, true, 0),
                                    span_of(c, 4 * nklq_packed_words(n_rows, n_cols), false)};
         if (spans_conflict(spans)) return NKLQ_EALIAS;
     }
@@ -1576,7 +1578,7 @@ int nklq_dequant_accumulate_f32(float* acc, const uint32_t* const* payloads, int
     if (!acc || !payloads) return NKLQ_ENULL;
     if (!aligned4(acc)) return NKLQ_EALIGN;
     {
-        std::vector<Span> spans = {span_of(acc, 4 * n, true)};
+        std::vector<Span> spans = {span_of(acc, 4 * n, true, 0)};
         for (int p = 0; p < k_payloads; ++p) {
             if (!payloads[p]) return NKLQ_ENULL;
             if (!aligned4(payloads[p])) return NKLQ_EALIGN;
@@ -1622,9 +1624,9 @@ int nklq_quantize_multi_f32(int count, const float* const* g, float* const* r, u
         spans.reserve(3 * (size_t)count);
         for (int i = 0; i < count; ++i) {
             if (n[i] == 0) continue;
-            spans.push_back(span_of(r[i], 4 * n[i], true));
-            spans.push_back(span_of(c[i], 4 * nklq_packed_words(n[i], 1), true));
-            spans.push_back(span_of(g[i], 4 * n[i], false));
+            spans.push_back(span_of(r[i], 4 * n[i], true, 2 * i));  // r[i] is its own input: in place
+            spans.push_back(span_of(c[i], 4 * nklq_packed_words(n[i], 1), true, 2 * i + 1));
+            spans.push_back(span_of(g[i], 4 * n[i], false, 2 * i));
         }
         if (spans_conflict(spans)) return NKLQ_EALIAS;
     }
@@ -1686,7 +1688,7 @@ int nklq_dequant_accumulate_multi_f32(int count, float* const* acc, const uint64
         spans.reserve((size_t)count + (size_t)k_payloads);
         for (int i = 0; i < count; ++i) {
             if (n[i] == 0) continue;
-            spans.push_back(span_of(acc[i], 4 * n[i], true));
+            spans.push_back(span_of(acc[i], 4 * n[i], true, i));
             if (word_offset[i] < w_lo) w_lo = word_offset[i];
             const uint64_t end = word_offset[i] + nklq_packed_words(n[i], 1);
             if (end > w_hi) w_hi = end;
@@ -1745,7 +1747,7 @@ int nklq_copy_f32(float* dst, const float* src, uint64_t n, void* stream)
     if (!dst || !src) return NKLQ_ENULL;
     if (!aligned16(dst) || !aligned16(src)) return NKLQ_EALIGN;
     {
-        std::vector<Span> spans = {span_of(dst, 4 * n, true), span_of(src, 4 * n, false)};
+        std::vector<Span> spans = {span_of(dst, 4 * n, true, 0), span_of(src, 4 * n, false)};
         if (spans_conflict(spans)) return NKLQ_EALIAS;
     }
     snapshot_knobs();

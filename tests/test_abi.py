@@ -84,6 +84,17 @@ def test_partial_overlaps_are_refused_without_a_launch():
     assert L.nklq_dequantize_f32(g, g + 4 * (n - 1), n, 1, 0.5, None) == -4     # words start inside out
     arr = (vp * 2)(c, g + 64)
     assert L.nklq_dequant_accumulate_f32(g, arr, 2, n, 0.5, 0, None) == -4      # second payload inside acc
+    # one row: as many code words as elements, so c can coincide exactly with an input; only the
+    # residual output has in-place partners (r_in, g)
+    q1 = lambda g_, rin, rout, c_: L.nklq_quantize_f32(g_, rin, rout, c_, 1, n, 0.5, 1, None)
+    assert q1(g, r, r, g) == -4                     # code words exactly on top of the gradient
+    assert q1(g, r, c, r) == -4                     # code words exactly on top of the residual input
+    assert q1(g, r, c, c) == -4                     # the two outputs on top of each other
+    assert L.nklq_dequantize_f32(g, g, 1, n, 0.5, None) == -4                   # floats written over their own words
+    arr1 = (vp * 1)(g)
+    assert L.nklq_dequant_accumulate_f32(g, arr1, 1, 1, 0.5, 1, None) == -4     # one element, one word, same place
+    gs1, rs1, cs1, ns1 = (vp * 1)(g), (vp * 1)(r), (vp * 1)(g), (u64 * 1)(1)
+    assert L.nklq_quantize_multi_f32(1, gs1, rs1, cs1, ns1, 0.5, 1, None) == -4  # c[0] == g[0], one element
     # many vectors: an output of one vector on top of a buffer of another
     gs, rs, cs = (vp * 2)(g, g + 0x4000), (vp * 2)(r, r + 0x4000), (vp * 2)(c, r + 0x4000 - 16)
     ns = (u64 * 2)(n, n)
