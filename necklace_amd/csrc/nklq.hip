@@ -664,9 +664,18 @@ __global__ __launch_bounds__(kRowsBlock) void deq_2d_rows_kernel(
         v.w = deq_code((w3 >> sh) & 3u, t);
         st4<true, NT>(orow + y, v);  // 16-byte aligned in both forms
     } else {
+        // a quad cut by an end of the row: its words are requested together (column clamped into the
+        // row) and then stored one by one; load - store - load - store would be four memory round
+        // trips in a row, and a wave lives about as long as its round trips take
+        uint32_t w[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int64_t yj = y + j < 0 ? 0 : (y + j < (int64_t)k ? y + j : (int64_t)k - 1);
+            w[j] = cw[yj];
+        }
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-            if (y + j >= 0 && y + j < (int64_t)k) orow[y + j] = deq_code((cw[y + j] >> sh) & 3u, t);
+            if (y + j >= 0 && y + j < (int64_t)k) orow[y + j] = deq_code((w[j] >> sh) & 3u, t);
     }
 }
 
@@ -690,7 +699,14 @@ constexpr uint64_t kBandsMaxColumns = 384;  // LDS words per workgroup; wider ma
 // (0.62-0.93) and keep those shapes.
 constexpr uint64_t kBandsMaxColumnsDecode = 800;
 constexpr uint64_t kBandsRangeQuant = 2048;   // elements per workgroup when bands are short: quantize
-constexpr uint64_t kBandsRangeDecode = 4096;  // and decode (measured)
+constexpr uint64_t kBandsDecodeElems = 960;      // decode: elements per workgroup, at least (about one quad per lane)
+constexpr uint64_t kBandsDecodeWholeMax = 1536;  // whole bands up to this many elements; longer ones are cut into runs of rows
+constexpr int kBandsDecodeRoundsRun = 4;         // a run of rows: the band's k <= 800 words over 256 lanes
+// words of a workgroup of whole bands: k of one band of at least kBandsDecodeElems elements, or fewer than
+// 2 * kBandsDecodeElems / 16 of several shorter ones
+static_assert(kBandsDecodeWholeMax / 16 <= (uint64_t)kBandsBlock && 2 * (kBandsDecodeElems / 16) <= (uint64_t)kBandsBlock,
+              "words of whole bands: one per lane");
+static_assert(kBandsMaxColumnsDecode <= (uint64_t)kBandsDecodeRoundsRun * kBandsBlock, "words of one band per workgroup");
 
 // (row within the workgroup's range, column) of local element index li; inv = floor(2^32 / k) + 1,
 // exact for li * k < 2^32 (li < 16384, k <= 1024 here).
@@ -793,56 +809,162 @@ __global__ __launch_bounds__(kBandsBlock) void quant_bands_kernel(
     for (uint32_t w = threadIdx.x; w < n_words; w += kBandsBlock) cq[w] = words[w];
 }
 
+// Decode of bands.  What the write stream to HBM wants decided the shape (all measured):
+//   * a workgroup writes a little over 4 KiB and ends, and workgroup i writes the i-th piece: the
+//     chip then sweeps the matrix as one narrow front, like the flat decode.  With 2, 4, 8 stores
+//     per lane (8 to 32 KiB per workgroup) the same stores ran at 0.81, 0.80, 0.75 of the HBM peak
+//     where one store per lane runs at 0.89;
+//   * with so little to do a workgroup lives about as long as its chain of dependent steps takes
+//     (arguments, code words, LDS, barrier, store), and the rate is the bytes of the resident
+//     workgroups over that time: every step added to the chain shows (a second round trip to memory
+//     behind the first cost 20 %, a few dozen scalar instructions of index arithmetic 5-15 %).  So
+//     the code words are requested at once, one per lane, and everything that can be worked out on
+//     the host is.
+// A workgroup's elements are whole rows, contiguous in memory: `bands_per_wg` whole bands here, or a
+// run of rows of ONE band in deq_band_runs_kernel when a band is longer than a workgroup's share.
+//
+// A lane decodes the rows of ITS word with immediate shifts (no row or column arithmetic per
+// element) and writes the floats into the range's image in LDS, `k` floats apart; lanes with
+// neighbouring words write neighbouring floats, so the writes are free of bank conflicts.  After a
+// barrier the image leaves as 16-byte quads laid out from a 16-byte boundary of `out` (LDS reads of
+// 16 bytes per lane, stores of 1 KiB per wave); only the first and the last quad of a range can be
+// partial.
+//
+// MIX: (+t, -t, +0) = h * th with th = -t/2 and h in {-2, +2, -0} taken from the recoded word as IEEE
+// halves, two elements per shift-and-mask (see acc_tile); the addend -0 keeps every result exact,
+// also -t = -0 for t = +0.  Any other t takes compare-and-select.
 template <bool NT>
+__device__ __forceinline__ void band_image_out(const float* band_image, float* oq, uint32_t a, uint32_t len)
+{
+    for (int32_t li = -(int32_t)a + 4 * (int32_t)threadIdx.x; li < (int32_t)len; li += 4 * kBandsBlock) {
+        f32x4 v = *reinterpret_cast<const f32x4*>(band_image + (li + (int32_t)a));
+        asm volatile("" : "+v"(v));  // keeps the load one 16-byte LDS read (element uses below would split it)
+        if (li >= 0 && li + 4 <= (int32_t)len) {
+            st4<true, NT>(oq + li, v);
+        } else {
+            const float e[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (li + j >= 0 && li + j < (int32_t)len) oq[li + j] = e[j];
+        }
+    }
+}
+
+template <bool NT, bool MIX>
 __global__ __launch_bounds__(kBandsBlock) void deq_bands_kernel(
     float* out, const uint32_t* __restrict__ c, uint64_t n, uint32_t k, uint32_t bands_per_wg, uint32_t inv,
-    float t)
+    float t, float th)
 {
-    __shared__ uint32_t words[kBandsMaxColumnsDecode];
+    extern __shared__ __attribute__((aligned(16))) float band_image_base[];  // 4 + bands_per_wg * 16 * k floats
+    float* band_image = static_cast<float*>(__builtin_assume_aligned(band_image_base, 16));
     const uint64_t m = (n + 15) / 16;
-    const uint64_t x0 = (uint64_t)blockIdx.x * bands_per_wg;  // (runs per XCD measured slower for the decode)
+    const uint64_t x0 = (uint64_t)blockIdx.x * bands_per_wg;
     const uint64_t x1 = (x0 + bands_per_wg < m) ? x0 + bands_per_wg : m;
     const uint64_t e0 = x0 * 16 * k;
     const uint64_t e1 = (x1 * 16 < n ? x1 * 16 : n) * k;
-    const uint32_t n_words = (uint32_t)(x1 - x0) * k;
-    const uint32_t len = (uint32_t)(e1 - e0);
-    const uint32_t* cq = c + x0 * k;
-    for (uint32_t w = threadIdx.x; w < n_words; w += kBandsBlock) words[w] = cq[w];
-    __syncthreads();
-    const uint32_t a = (uint32_t)((reinterpret_cast<uintptr_t>(out + e0) >> 2) & 3u);
+    const uint32_t n_words = (uint32_t)(x1 - x0) * k;  // at most kBandsBlock: one per lane
     float* oq = out + e0;
-    for (int32_t li = -(int32_t)a + 4 * (int32_t)threadIdx.x; li < (int32_t)len; li += 4 * kBandsBlock) {
-        uint32_t row, col;
-        band_row_col((uint32_t)(li < 0 ? 0 : li), k, inv, &row, &col);
-        if (li >= 0 && li + 4 <= (int32_t)len) {
-            // a whole quad (all but the first and last of a range): no bounds to check
-            f32x4 vo;
-            if (col + 4 <= k) {
-                // inside one row, the usual case: one word address and one bit position for all four
-                const uint32_t* wq = &words[(row >> 4) * k + col];
-                const uint32_t sh = 2 * (row & 15u);
-                vo.x = deq_code((wq[0] >> sh) & 3u, t);
-                vo.y = deq_code((wq[1] >> sh) & 3u, t);
-                vo.z = deq_code((wq[2] >> sh) & 3u, t);
-                vo.w = deq_code((wq[3] >> sh) & 3u, t);
-            } else {
-                float o[4];
+    // element li of the range lives at band_image[a + li]: quads that start on a 16-byte boundary of
+    // `out` then start on one of the image
+    const uint32_t a = (uint32_t)((reinterpret_cast<uintptr_t>(oq) >> 2) & 3u);
+    const uint32_t w = threadIdx.x;
+    if (w < n_words) {
+        uint32_t b = 0, y = w;
+        if (bands_per_wg > 1) band_row_col(w, k, inv, &b, &y);  // band within the range, column
+        const uint32_t word = c[x0 * k + w];
+        float* col = band_image + a + b * 16 * k + y;
+        if constexpr (MIX) {
+            const uint32_t tops = codes_to_half_tops(word);
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    o[j] = deq_code((words[(row >> 4) * k + col] >> (2 * (row & 15u))) & 3u, t);
-                    if (++col == k) { col = 0; ++row; }
-                }
-                vo.x = o[0]; vo.y = o[1]; vo.z = o[2]; vo.w = o[3];
+            for (int s = 0; s < 8; ++s) {
+                const f16x2 h = __builtin_bit_cast(f16x2, (tops << (14 - 2 * s)) & 0xC000C000u);
+                col[s * k] = __builtin_fmaf((float)h.x, th, -0.0f);
+                col[(s + 8) * k] = __builtin_fmaf((float)h.y, th, -0.0f);
             }
-            st4<true, NT>(oq + li, vo);
         } else {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                if (li + j >= 0 && li + j < (int32_t)len) {
-                    oq[li + j] = deq_code((words[(row >> 4) * k + col] >> (2 * (row & 15u))) & 3u, t);
-                    if (++col == k) { col = 0; ++row; }
-                }
-            }
+            for (int s = 0; s < 16; ++s) col[s * k] = deq_code((word >> (2 * s)) & 3u, t);
+        }
+    }
+    __syncthreads();
+    band_image_out<NT>(band_image, oq, a, (uint32_t)(e1 - e0));
+}
+
+// Bands longer than that (97 to 800 columns).  The band is cut into 2^gs runs of 16 >> gs rows (900
+// to 1800 elements each), workgroup (band, g) takes run g.  Here a lane per word would leave most
+// lanes idle and one lane with a long chain of its own, so the work is turned round: the band's words
+// go to LDS as they are (one step: load, store, barrier), and every lane decodes the quad IT stores:
+// (row, column) of the quad by one multiply-high, its four words by ONE 16-byte LDS read, one bit
+// position for all four.  The words are kept four times, copy p shifted so that the words whose
+// column is p modulo 4 sit on 16-byte boundaries: a quad then reads copy (column mod 4) aligned, and
+// neighbouring lanes read neighbouring 16 bytes (no bank conflicts; one copy read at stride 4 words
+// put 32 lanes on 8 banks).  A quad that runs over the end of its row takes its last elements from
+// the first words of the next row, read by every lane and selected without a branch.
+// The 2^gs workgroups of a band all read its words; they run on ONE XCD (workgroups go to the XCDs
+// round-robin by id: bands are dealt to the XCDs in groups of 8), so the words come from memory once.
+constexpr uint32_t kRunsCopyWords = kBandsMaxColumnsDecode + 8;  // words of one copy (a multiple of 4), with slack for the shift
+
+template <bool NT>
+__global__ __launch_bounds__(kBandsBlock) void deq_band_runs_kernel(
+    float* out, const uint32_t* __restrict__ c, uint64_t n, uint32_t k, uint32_t gs, uint32_t inv, float t)
+{
+    __shared__ __attribute__((aligned(16))) uint32_t words[4 * kRunsCopyWords];
+    const uint32_t xcd = blockIdx.x & 7u, j = blockIdx.x >> 3;
+    const uint64_t x = (uint64_t)(j >> gs) * 8 + xcd;
+    const uint32_t rows = 16u >> gs;
+    const uint32_t ra = (j & ((1u << gs) - 1u)) * rows;
+    const uint64_t row0 = x * 16 + ra;
+    if (row0 >= n) return;  // rows past the end of the matrix, padding workgroups of the last 8 bands
+    const uint32_t len = (uint32_t)(row0 + rows <= n ? rows : n - row0) * k;
+    const uint32_t* cq = c + x * k;
+    float* oq = out + row0 * k;
+    uint32_t wd[kBandsDecodeRoundsRun];
+#pragma unroll
+    for (int r = 0; r < kBandsDecodeRoundsRun; ++r) {
+        const uint32_t w = threadIdx.x + kBandsBlock * r;
+        wd[r] = w < k ? cq[w] : 0u;
+    }
+#pragma unroll
+    for (int r = 0; r < kBandsDecodeRoundsRun; ++r) {
+        const uint32_t w = threadIdx.x + kBandsBlock * r;
+        if (w < k) {
+            // copy p holds word w at p * kRunsCopyWords + 4 + w - p  (p = 0..3)
+#pragma unroll
+            for (uint32_t p = 0; p < 4; ++p) words[p * (kRunsCopyWords - 1) + 4 + w] = wd[r];
+        }
+    }
+    __syncthreads();
+    const uint32_t a = (uint32_t)((reinterpret_cast<uintptr_t>(oq) >> 2) & 3u);
+    for (int32_t li = -(int32_t)a + 4 * (int32_t)threadIdx.x; li < (int32_t)len; li += 4 * kBandsBlock) {
+        // (row, col) of the quad's first element; counted from one row before the run so that the first
+        // quad, which may start up to 3 elements before it, needs no case of its own
+        uint32_t row1, col;
+        band_row_col((uint32_t)(li + (int32_t)k), k, inv, &row1, &col);
+        const uint32_t sh = 2 * (ra + row1) - 2;  // bit position of this row's codes (of no use for row1 = 0: never stored)
+        // words of columns col .. col+3 of this row (the ones past its end are not used) and of columns
+        // 0 .. 3 of the next row: two aligned 16-byte reads, the second from the same place for every lane
+        const uint32_t p = col & 3u;
+        const u32x4 wa = *reinterpret_cast<const u32x4*>(&words[p * kRunsCopyWords + 4 + (col - p)]);
+        const u32x4 wb = *reinterpret_cast<const u32x4*>(&words[4]);
+        const uint32_t nf = k - col;  // elements of the quad that lie in this row (4 or more: all)
+        const uint32_t sa = sh & 31u, sb = (sh + 2) & 31u;
+        const uint32_t a0 = wa.x >> sa, a1 = wa.y >> sa, a2 = wa.z >> sa, a3 = wa.w >> sa;
+        const uint32_t b0 = wb.x >> sb, b1 = wb.y >> sb, b2 = wb.z >> sb;
+        const uint32_t c1 = nf > 1 ? a1 : b0;
+        const uint32_t c2 = nf > 2 ? a2 : (nf == 2 ? b0 : b1);
+        const uint32_t c3 = nf > 3 ? a3 : (nf == 3 ? b0 : (nf == 2 ? b1 : b2));
+        f32x4 vo;
+        vo.x = deq_code(a0 & 3u, t);
+        vo.y = deq_code(c1 & 3u, t);
+        vo.z = deq_code(c2 & 3u, t);
+        vo.w = deq_code(c3 & 3u, t);
+        if (li >= 0 && li + 4 <= (int32_t)len) {
+            st4<true, NT>(oq + li, vo);
+        } else {
+            const float o[4] = {vo.x, vo.y, vo.z, vo.w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (li + e >= 0 && li + e < (int32_t)len) oq[li + e] = o[e];
         }
     }
 }
@@ -1540,17 +1662,43 @@ int nklq_dequantize_f32(float* out, const uint32_t* c, uint64_t n_rows, uint64_t
     const uint64_t m = n_rows / 16 + (n_rows % 16 ? 1 : 0);
     if (n_cols <= kBandsMaxColumns ||
         (n_cols <= kBandsMaxColumnsDecode && (n_cols % 2 != 0 || !aligned16(out)))) {
-        uint32_t per;
-        const uint32_t grid = bands_grid(n_rows, n_cols, kBandsRangeDecode, false, &per);
-        if (grid == 0) return NKLQ_ERANGE;
+        // whole bands while they are short (the fewest that give every lane of the workgroup a quad), else
+        // runs of at least kBandsDecodeElems / k rows of one band
         const uint32_t k32 = (uint32_t)n_cols;
-        const uint32_t inv = (uint32_t)(0x100000000ull / k32) + 1u;
-        if (tk.nontemporal)
-            launch_kernel((deq_bands_kernel<true>), dim3(grid), dim3(kBandsBlock), 0, s, out, c, n_rows,
-                               k32, per, inv, thrd);
-        else
-            launch_kernel((deq_bands_kernel<false>), dim3(grid), dim3(kBandsBlock), 0, s, out, c, n_rows,
-                               k32, per, inv, thrd);
+        const bool mix = mix_ok(thrd);
+        const float th = -0.5f * thrd;
+        if (16 * n_cols <= kBandsDecodeWholeMax) {
+            const uint32_t inv = (uint32_t)(0x100000000ull / k32) + 1u;
+            const uint32_t per = (uint32_t)((kBandsDecodeElems + 16 * n_cols - 1) / (16 * n_cols));
+            const uint64_t blocks = (m + per - 1) / per;
+            if (blocks > 0x7FFFFFFFull) return NKLQ_ERANGE;
+            const uint32_t lds = 4u * (4u + 16u * per * k32);
+#define NKLQ_DB(NT, MIX)                                                                                      \
+    launch_kernel((deq_bands_kernel<NT, MIX>), dim3((uint32_t)blocks), dim3(kBandsBlock), lds, s, out, c, n_rows, \
+                  k32, per, inv, thrd, th)
+            if (tk.nontemporal && mix) NKLQ_DB(true, true);
+            else if (tk.nontemporal) NKLQ_DB(true, false);
+            else if (mix) NKLQ_DB(false, true);
+            else NKLQ_DB(false, false);
+#undef NKLQ_DB
+        } else {
+            // the most runs per band that still have kBandsDecodeElems elements each.  When rows are not
+            // whole quads, only runs that leave in ONE round of stores measured faster than the whole band
+            // (0.82-0.83 of the HBM peak against 0.73-0.78 at 127 and 255 columns; runs of 1600 elements
+            // 0.60-0.69 against 0.64-0.77 at 201, 385, 401, 799 columns)
+            uint32_t gs = 0;
+            while (gs < 3 && (16u >> (gs + 1)) * n_cols >= kBandsDecodeElems) ++gs;
+            if (n_cols % 4 != 0 && (16u >> gs) * n_cols > kBandsDecodeElems + 160) gs = 0;
+            const uint64_t blocks = ((m + 7) / 8 * 8) << gs;
+            if (blocks > 0x7FFFFFFFull) return NKLQ_ERANGE;
+            const uint32_t inv = (uint32_t)(0x100000000ull / k32) + 1u;
+            if (tk.nontemporal)
+                launch_kernel((deq_band_runs_kernel<true>), dim3((uint32_t)blocks), dim3(kBandsBlock), 0, s, out, c,
+                              n_rows, k32, gs, inv, thrd);
+            else
+                launch_kernel((deq_band_runs_kernel<false>), dim3((uint32_t)blocks), dim3(kBandsBlock), 0, s, out, c,
+                              n_rows, k32, gs, inv, thrd);
+        }
         return launch_status();
     }
     // rows that all start on a 128-byte line (and 16-byte aligned words) take the plain form
