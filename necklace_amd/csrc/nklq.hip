@@ -692,21 +692,13 @@ __global__ __launch_bounds__(kRowsBlock) void deq_2d_rows_kernel(
 // LDS; after a barrier the words are stored, contiguous.
 constexpr int kBandsBlock = 256;
 constexpr uint64_t kBandsMaxColumns = 384;  // LDS words per workgroup; wider matrices take the row tiles (measured crossover: 300-500 columns)
-// The decode also takes bands for up to 800 columns when most rows start off a 16-byte boundary
-// (an odd k, or a base off one): the row tiles then cut a quad at both ends of nearly every row
-// and measured 0.45-0.60 of the HBM peak at 385..799 columns against 0.60-0.67 here; with whole
-// quads in every row, or every other row (k = 2 mod 4), the row tiles are as fast or faster
-// (0.62-0.93) and keep those shapes.
-constexpr uint64_t kBandsMaxColumnsDecode = 800;
-constexpr uint64_t kBandsRangeQuant = 2048;   // elements per workgroup when bands are short: quantize
+constexpr uint64_t kBandsRangeQuant = 2048;      // elements per workgroup when bands are short: quantize
 constexpr uint64_t kBandsDecodeElems = 960;      // decode: elements per workgroup, at least (about one quad per lane)
-constexpr uint64_t kBandsDecodeWholeMax = 1536;  // whole bands up to this many elements; longer ones are cut into runs of rows
-constexpr int kBandsDecodeRoundsRun = 4;         // a run of rows: the band's k <= 800 words over 256 lanes
+constexpr uint64_t kBandsDecodeWholeMax = 1536;  // decode: bands up to this many elements (96 columns) go through the LDS image
 // words of a workgroup of whole bands: k of one band of at least kBandsDecodeElems elements, or fewer than
 // 2 * kBandsDecodeElems / 16 of several shorter ones
 static_assert(kBandsDecodeWholeMax / 16 <= (uint64_t)kBandsBlock && 2 * (kBandsDecodeElems / 16) <= (uint64_t)kBandsBlock,
               "words of whole bands: one per lane");
-static_assert(kBandsMaxColumnsDecode <= (uint64_t)kBandsDecodeRoundsRun * kBandsBlock, "words of one band per workgroup");
 
 // (row within the workgroup's range, column) of local element index li; inv = floor(2^32 / k) + 1,
 // exact for li * k < 2^32 (li < 16384, k <= 1024 here).
@@ -820,8 +812,8 @@ __global__ __launch_bounds__(kBandsBlock) void quant_bands_kernel(
 //     behind the first cost 20 %, a few dozen scalar instructions of index arithmetic 5-15 %).  So
 //     the code words are requested at once, one per lane, and everything that can be worked out on
 //     the host is.
-// A workgroup's elements are whole rows, contiguous in memory: `bands_per_wg` whole bands here, or a
-// run of rows of ONE band in deq_band_runs_kernel when a band is longer than a workgroup's share.
+// A workgroup's elements are whole rows, contiguous in memory: `bands_per_wg` whole bands;
+// for longer bands see deq_stream_kernel.
 //
 // A lane decodes the rows of ITS word with immediate shifts (no row or column arithmetic per
 // element) and writes the floats into the range's image in LDS, `k` floats apart; lanes with
@@ -890,82 +882,71 @@ __global__ __launch_bounds__(kBandsBlock) void deq_bands_kernel(
     band_image_out<NT>(band_image, oq, a, (uint32_t)(e1 - e0));
 }
 
-// Bands longer than that (97 to 800 columns).  The band is cut into 2^gs runs of 16 >> gs rows (900
-// to 1800 elements each), workgroup (band, g) takes run g.  Here a lane per word would leave most
-// lanes idle and one lane with a long chain of its own, so the work is turned round: the band's words
-// go to LDS as they are (one step: load, store, barrier), and every lane decodes the quad IT stores:
-// (row, column) of the quad by one multiply-high, its four words by ONE 16-byte LDS read, one bit
-// position for all four.  The words are kept four times, copy p shifted so that the words whose
-// column is p modulo 4 sit on 16-byte boundaries: a quad then reads copy (column mod 4) aligned, and
-// neighbouring lanes read neighbouring 16 bytes (no bank conflicts; one copy read at stride 4 words
-// put 32 lanes on 8 banks).  A quad that runs over the end of its row takes its last elements from
-// the first words of the next row, read by every lane and selected without a branch.
-// The 2^gs workgroups of a band all read its words; they run on ONE XCD (workgroups go to the XCDs
-// round-robin by id: bands are dealt to the XCDs in groups of 8), so the words come from memory once.
-constexpr uint32_t kRunsCopyWords = kBandsMaxColumnsDecode + 8;  // words of one copy (a multiple of 4), with slack for the shift
+// Bands longer than that: no LDS and no barrier at all.  A band (16 rows of the matrix, 16 k contiguous
+// floats, k code words) is cut on a grid of 4 KiB pieces that starts at the 128-byte line at or
+// before the band: workgroup (band, piece) writes one piece, a wave 1 KiB of whole lines, a lane one
+// quad, exactly like the flat decode.  The lane finds (row, column) of its quad by one multiply-high
+// and fetches the four words of columns col .. col+3 with ONE 16-byte load at word alignment;
+// neighbouring lanes read neighbouring 16 bytes, so a wave reads 1 KiB of contiguous words.  A quad
+// that runs over the end of its row takes its last elements from the first words of the band (the
+// next row's), which every lane loads from the same address; the four words are picked out of the
+// seven without a branch.  Each word is read by the 16 waves that write its 16 rows: the workgroups
+// of a band run on ONE XCD (workgroups go to the XCDs round-robin by id; bands are dealt to the XCDs
+// in groups of 8), so it comes from memory once and from that XCD's L2 fifteen times (measured at 401
+// columns: 0.83 of the HBM peak with the bands pinned, 0.70 in plain order).
+// Measured against what it replaced (band kernels with the words staged in LDS up to 800 columns,
+// tiles of 16 rows x 256 columns above): 0.83 against 0.68 at 401 columns, 0.88 / 0.70 at 201,
+// 0.95 / 0.80 at 255, 0.79 / 0.65 at 799, 0.85 / 0.67 at 1001, 0.96 / 0.89 at 8191.
+// For 97 to 8192 columns (the 32-bit multiply-high is exact while 17 k^2 + 1024 k < 2^32); wider matrices
+// keep the tiles of 16 rows x 256 columns.
+constexpr uint64_t kStreamMaxColumns = 8192;
 
 template <bool NT>
-__global__ __launch_bounds__(kBandsBlock) void deq_band_runs_kernel(
-    float* out, const uint32_t* __restrict__ c, uint64_t n, uint32_t k, uint32_t gs, uint32_t inv, float t)
+__global__ __launch_bounds__(256) void deq_stream_kernel(
+    float* out, const uint32_t* __restrict__ c, uint64_t n, uint32_t k, uint32_t pieces, uint64_t inv_pieces,
+    uint32_t inv_k, float t)
 {
-    __shared__ __attribute__((aligned(16))) uint32_t words[4 * kRunsCopyWords];
     const uint32_t xcd = blockIdx.x & 7u, j = blockIdx.x >> 3;
-    const uint64_t x = (uint64_t)(j >> gs) * 8 + xcd;
-    const uint32_t rows = 16u >> gs;
-    const uint32_t ra = (j & ((1u << gs) - 1u)) * rows;
-    const uint64_t row0 = x * 16 + ra;
-    if (row0 >= n) return;  // rows past the end of the matrix, padding workgroups of the last 8 bands
-    const uint32_t len = (uint32_t)(row0 + rows <= n ? rows : n - row0) * k;
+    const uint32_t jb = (uint32_t)__umul64hi((uint64_t)j, inv_pieces);  // j / pieces
+    const uint32_t q = j - jb * pieces;                                 // piece within the band
+    const uint64_t x = (uint64_t)jb * 8 + xcd;                          // band
+    if (x * 16 >= n) return;  // padding workgroups of the last group of 8 bands
+    const uint32_t rows = n - x * 16 < 16 ? (uint32_t)(n - x * 16) : 16u;
+    const int32_t blen = (int32_t)(rows * k);
+    float* ob = out + x * 16 * k;
     const uint32_t* cq = c + x * k;
-    float* oq = out + row0 * k;
-    uint32_t wd[kBandsDecodeRoundsRun];
+    const int32_t d = (int32_t)((reinterpret_cast<uintptr_t>(ob) >> 2) & 31u);
+    const int32_t li = 1024 * (int32_t)q - d + 4 * (int32_t)threadIdx.x;  // first element of the quad, within the band
+    if (li + 4 <= 0 || li >= blen) return;
+    // (row, col), counted from one row before the band so that a first quad that starts before it
+    // needs no case of its own: its elements inside the band are "the next row's"
+    const uint32_t v = (uint32_t)(li + (int32_t)k);
+    const uint32_t row1 = __umulhi(v, inv_k);
+    const uint32_t col = v - row1 * k;
+    const uint32_t sh = 2 * row1 - 2;               // bit position of this row's codes (of no use for row1 = 0: never stored)
+    const uint32_t nf = k - col;                    // elements of the quad that lie in this row (4 or more: all)
+    const uint32_t col_a = nf >= 4 ? col : k - 4;   // the load stays inside the band's words
+    const u32x4_a4 wa = *reinterpret_cast<const u32x4_a4*>(cq + col_a);
+    const u32x4_a4 wb = *reinterpret_cast<const u32x4_a4*>(cq);
+    const uint32_t first = nf >= 4 ? 0u : 4u - nf;  // the quad's words are v[first .. first + 3]
+    const uint32_t sa = sh & 31u, sb = (sh + 2) & 31u;
+    const uint32_t v0 = wa.x >> sa, v1 = wa.y >> sa, v2 = wa.z >> sa, v3 = wa.w >> sa;
+    const uint32_t v4 = wb.x >> sb, v5 = wb.y >> sb, v6 = wb.z >> sb;
+    const bool f1 = first & 1u, f2 = first & 2u;
+    const uint32_t y0 = f1 ? v1 : v0, y1 = f1 ? v2 : v1, y2 = f1 ? v3 : v2, y3 = f1 ? v4 : v3, y4 = f1 ? v5 : v4,
+                   y5 = f1 ? v6 : v5;
+    f32x4 vo;
+    vo.x = deq_code((f2 ? y2 : y0) & 3u, t);
+    vo.y = deq_code((f2 ? y3 : y1) & 3u, t);
+    vo.z = deq_code((f2 ? y4 : y2) & 3u, t);
+    vo.w = deq_code((f2 ? y5 : y3) & 3u, t);
+    if (li >= 0 && li + 4 <= blen) {
+        st4<true, NT>(ob + li, vo);
+    } else {
+        const float o[4] = {vo.x, vo.y, vo.z, vo.w};
 #pragma unroll
-    for (int r = 0; r < kBandsDecodeRoundsRun; ++r) {
-        const uint32_t w = threadIdx.x + kBandsBlock * r;
-        wd[r] = w < k ? cq[w] : 0u;
-    }
-#pragma unroll
-    for (int r = 0; r < kBandsDecodeRoundsRun; ++r) {
-        const uint32_t w = threadIdx.x + kBandsBlock * r;
-        if (w < k) {
-            // copy p holds word w at p * kRunsCopyWords + 4 + w - p  (p = 0..3)
-#pragma unroll
-            for (uint32_t p = 0; p < 4; ++p) words[p * (kRunsCopyWords - 1) + 4 + w] = wd[r];
-        }
-    }
-    __syncthreads();
-    const uint32_t a = (uint32_t)((reinterpret_cast<uintptr_t>(oq) >> 2) & 3u);
-    for (int32_t li = -(int32_t)a + 4 * (int32_t)threadIdx.x; li < (int32_t)len; li += 4 * kBandsBlock) {
-        // (row, col) of the quad's first element; counted from one row before the run so that the first
-        // quad, which may start up to 3 elements before it, needs no case of its own
-        uint32_t row1, col;
-        band_row_col((uint32_t)(li + (int32_t)k), k, inv, &row1, &col);
-        const uint32_t sh = 2 * (ra + row1) - 2;  // bit position of this row's codes (of no use for row1 = 0: never stored)
-        // words of columns col .. col+3 of this row (the ones past its end are not used) and of columns
-        // 0 .. 3 of the next row: two aligned 16-byte reads, the second from the same place for every lane
-        const uint32_t p = col & 3u;
-        const u32x4 wa = *reinterpret_cast<const u32x4*>(&words[p * kRunsCopyWords + 4 + (col - p)]);
-        const u32x4 wb = *reinterpret_cast<const u32x4*>(&words[4]);
-        const uint32_t nf = k - col;  // elements of the quad that lie in this row (4 or more: all)
-        const uint32_t sa = sh & 31u, sb = (sh + 2) & 31u;
-        const uint32_t a0 = wa.x >> sa, a1 = wa.y >> sa, a2 = wa.z >> sa, a3 = wa.w >> sa;
-        const uint32_t b0 = wb.x >> sb, b1 = wb.y >> sb, b2 = wb.z >> sb;
-        const uint32_t c1 = nf > 1 ? a1 : b0;
-        const uint32_t c2 = nf > 2 ? a2 : (nf == 2 ? b0 : b1);
-        const uint32_t c3 = nf > 3 ? a3 : (nf == 3 ? b0 : (nf == 2 ? b1 : b2));
-        f32x4 vo;
-        vo.x = deq_code(a0 & 3u, t);
-        vo.y = deq_code(c1 & 3u, t);
-        vo.z = deq_code(c2 & 3u, t);
-        vo.w = deq_code(c3 & 3u, t);
-        if (li >= 0 && li + 4 <= (int32_t)len) {
-            st4<true, NT>(oq + li, vo);
-        } else {
-            const float o[4] = {vo.x, vo.y, vo.z, vo.w};
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-                if (li + e >= 0 && li + e < (int32_t)len) oq[li + e] = o[e];
-        }
+        for (int e = 0; e < 4; ++e)
+            if (li + e >= 0 && li + e < blen) ob[li + e] = o[e];
     }
 }
 
@@ -1660,61 +1641,58 @@ int nklq_dequantize_f32(float* out, const uint32_t* c, uint64_t n_rows, uint64_t
         return dispatch_deq_flat(out, c, total, thrd, s);
     }
     const uint64_t m = n_rows / 16 + (n_rows % 16 ? 1 : 0);
-    if (n_cols <= kBandsMaxColumns ||
-        (n_cols <= kBandsMaxColumnsDecode && (n_cols % 2 != 0 || !aligned16(out)))) {
-        // whole bands while they are short (the fewest that give every lane of the workgroup a quad), else
-        // runs of at least kBandsDecodeElems / k rows of one band
+    if (16 * n_cols <= kBandsDecodeWholeMax) {
+        // short bands: the fewest whole bands that give every lane of the workgroup a quad
         const uint32_t k32 = (uint32_t)n_cols;
         const bool mix = mix_ok(thrd);
         const float th = -0.5f * thrd;
-        if (16 * n_cols <= kBandsDecodeWholeMax) {
-            const uint32_t inv = (uint32_t)(0x100000000ull / k32) + 1u;
-            const uint32_t per = (uint32_t)((kBandsDecodeElems + 16 * n_cols - 1) / (16 * n_cols));
-            const uint64_t blocks = (m + per - 1) / per;
-            if (blocks > 0x7FFFFFFFull) return NKLQ_ERANGE;
-            const uint32_t lds = 4u * (4u + 16u * per * k32);
+        const uint32_t inv = (uint32_t)(0x100000000ull / k32) + 1u;
+        const uint32_t per = (uint32_t)((kBandsDecodeElems + 16 * n_cols - 1) / (16 * n_cols));
+        const uint64_t blocks = (m + per - 1) / per;
+        if (blocks > 0x7FFFFFFFull) return NKLQ_ERANGE;
+        const uint32_t lds = 4u * (4u + 16u * per * k32);
 #define NKLQ_DB(NT, MIX)                                                                                      \
     launch_kernel((deq_bands_kernel<NT, MIX>), dim3((uint32_t)blocks), dim3(kBandsBlock), lds, s, out, c, n_rows, \
                   k32, per, inv, thrd, th)
-            if (tk.nontemporal && mix) NKLQ_DB(true, true);
-            else if (tk.nontemporal) NKLQ_DB(true, false);
-            else if (mix) NKLQ_DB(false, true);
-            else NKLQ_DB(false, false);
+        if (tk.nontemporal && mix) NKLQ_DB(true, true);
+        else if (tk.nontemporal) NKLQ_DB(true, false);
+        else if (mix) NKLQ_DB(false, true);
+        else NKLQ_DB(false, false);
 #undef NKLQ_DB
-        } else {
-            // the most runs per band that still have kBandsDecodeElems elements each.  When rows are not
-            // whole quads, only runs that leave in ONE round of stores measured faster than the whole band
-            // (0.82-0.83 of the HBM peak against 0.73-0.78 at 127 and 255 columns; runs of 1600 elements
-            // 0.60-0.69 against 0.64-0.77 at 201, 385, 401, 799 columns)
-            uint32_t gs = 0;
-            while (gs < 3 && (16u >> (gs + 1)) * n_cols >= kBandsDecodeElems) ++gs;
-            if (n_cols % 4 != 0 && (16u >> gs) * n_cols > kBandsDecodeElems + 160) gs = 0;
-            const uint64_t blocks = ((m + 7) / 8 * 8) << gs;
-            if (blocks > 0x7FFFFFFFull) return NKLQ_ERANGE;
-            const uint32_t inv = (uint32_t)(0x100000000ull / k32) + 1u;
-            if (tk.nontemporal)
-                launch_kernel((deq_band_runs_kernel<true>), dim3((uint32_t)blocks), dim3(kBandsBlock), 0, s, out, c,
-                              n_rows, k32, gs, inv, thrd);
-            else
-                launch_kernel((deq_band_runs_kernel<false>), dim3((uint32_t)blocks), dim3(kBandsBlock), 0, s, out, c,
-                              n_rows, k32, gs, inv, thrd);
-        }
         return launch_status();
     }
-    // rows that all start on a 128-byte line (and 16-byte aligned words) take the plain form
+    // Tiles of 16 rows x 256 columns for more than 8192 columns (0.93 of the HBM peak against 0.86 for the band
+    // stream at 16384 x 16383) and from 4096 columns when every row starts on a 128-byte line (0.89 against 0.85
+    // at 8192 x 8192 in one process; the band stream is ahead at 1024 and 2048 columns, and at 8191: 0.96 / 0.89)
     const bool plain = (n_cols % 32 == 0) && (reinterpret_cast<uintptr_t>(out) & 127u) == 0 && aligned16(c);
-    const uint64_t col_tiles = ((plain ? n_cols : n_cols + 31) + 255) / 256;
-    const uint64_t m8 = (m + 7) / 8 * 8;  // word rows are dealt to the XCDs in groups of 8
-    if (col_tiles > 0x7FFFFFFFull || m8 > 0x7FFFFFFFull / col_tiles) return NKLQ_ERANGE;
-    const dim3 grid((uint32_t)(m8 * col_tiles)), block(kRowsBlock);
+    if (n_cols > kStreamMaxColumns || (n_cols >= 4096 && plain)) {
+        const uint64_t col_tiles = ((plain ? n_cols : n_cols + 31) + 255) / 256;
+        const uint64_t m8 = (m + 7) / 8 * 8;  // word rows are dealt to the XCDs in groups of 8
+        if (col_tiles > 0x7FFFFFFFull || m8 > 0x7FFFFFFFull / col_tiles) return NKLQ_ERANGE;
+        const dim3 grid((uint32_t)(m8 * col_tiles)), block(kRowsBlock);
 #define NKLQ_D2(NT, SHIFT)                                                                        \
     launch_kernel((deq_2d_rows_kernel<NT, SHIFT>), grid, block, 0, s, out, c, n_rows, n_cols, \
                        (uint32_t)col_tiles, thrd)
-    if (tk.nontemporal && plain) NKLQ_D2(true, false);
-    else if (tk.nontemporal) NKLQ_D2(true, true);
-    else if (plain) NKLQ_D2(false, false);
-    else NKLQ_D2(false, true);
+        if (tk.nontemporal && plain) NKLQ_D2(true, false);
+        else if (tk.nontemporal) NKLQ_D2(true, true);
+        else if (plain) NKLQ_D2(false, false);
+        else NKLQ_D2(false, true);
 #undef NKLQ_D2
+        return launch_status();
+    }
+    // everything else (97 .. 8192 columns): the band stream
+    const uint64_t pieces = (16 * n_cols + 31 + 1023) / 1024;  // 4 KiB pieces of a band, on a grid that starts up to 31 elements before it
+    const uint64_t m8 = (m + 7) / 8 * 8;
+    if (m8 > 0x7FFFFFFFull / pieces) return NKLQ_ERANGE;
+    const uint32_t blocks = (uint32_t)(m8 * pieces);
+    const uint64_t inv_pieces = ~0ull / pieces + 1;  // floor(2^64 / pieces) + 1 (pieces >= 2): exact quotients for j * pieces < 2^64
+    const uint32_t inv_k = (uint32_t)(0x100000000ull / n_cols) + 1u;
+    if (tk.nontemporal)
+        launch_kernel((deq_stream_kernel<true>), dim3(blocks), dim3(256), 0, s, out, c, n_rows, (uint32_t)n_cols,
+                      (uint32_t)pieces, inv_pieces, inv_k, thrd);
+    else
+        launch_kernel((deq_stream_kernel<false>), dim3(blocks), dim3(256), 0, s, out, c, n_rows, (uint32_t)n_cols,
+                      (uint32_t)pieces, inv_pieces, inv_k, thrd);
     return launch_status();
 }
 
