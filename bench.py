@@ -700,9 +700,18 @@ def main():
             gcomp.decompress_sum(outs)
         _, ev = time_region(torch, lambda: gcomp.compress(gl), 50)
         _, ev2 = time_region(torch, lambda: gcomp.decompress_sum(outs), 50)
+        # host side of a steady-state call (gradients keep their storage): wall time until the call
+        # returns, launches left in flight (200 calls stay far below the depth of the launch queue)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(200):
+            gcomp.compress(gl)
+        host_us = (time.perf_counter() - t0) / 200 * 1e6
+        torch.cuda.synchronize()
         res["resnet50_tensor_list"] = {
             "tensors": len(sizes), "compressed_elements": nel,
             "compress_us": round(ev / 50 * 1e3, 1), "decompress_sum_us": round(ev2 / 50 * 1e3, 1),
+            "host_us_per_call": round(host_us, 1),
         }
 
     if "copy" in legs:

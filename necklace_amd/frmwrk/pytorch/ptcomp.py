@@ -47,6 +47,24 @@ def _sync(device, stream):
         stream.synchronize()
 
 
+class _stream_ctx:
+    """`with torch.cuda.stream(s)` for a torch stream; nothing for None (the current stream is the
+    one) or a raw handle (torch cannot enter it: the caller orders such work itself)."""
+    __slots__ = ("ctx",)
+
+    def __init__(self, stream):
+        self.ctx = None if stream is None or isinstance(stream, int) else torch.cuda.stream(stream)
+
+    def __enter__(self):
+        if self.ctx is not None:
+            self.ctx.__enter__()
+
+    def __exit__(self, *exc):
+        if self.ctx is not None:
+            return self.ctx.__exit__(*exc)
+        return False
+
+
 def _numel(p):
     if isinstance(p, int):
         return p
@@ -122,39 +140,60 @@ class GradCompressor:
         # parameters that have a gradient)
         self._idx = [i for i, c in enumerate(self.grd_cmps) if c]
         self._live_key, self._live_tabs = None, None
+        self._addr_cache = {}
         # what Tensor.get_device() returns for tensors that live where the buffers do; host tensors
         # (-1) never match: there is no CPU path
         self._dev_index = self.resi.get_device() if self.resi.is_cuda else -2
         self._pl_arr = (ct.c_void_p * self.kn)(*[self.recv[k].data_ptr() for k in range(self.kn)])
 
-    def _tables(self, tensors, what):
+    def _tables(self, tensors, what, stream=None):
         """Argument tables for the compressed parameters whose tensor is present (not None) in this
-        call; cached while the same subset comes back.  Returns (count, ptrs, r, c, n, word_offset)."""
+        call.  Returns (count, ptrs, r, c, n, word_offset, staged); `staged` lists (tensor,
+        contiguous temporary) pairs for tensors that are not contiguous (their temporary is what the
+        kernels see).
+
+        Gradients normally keep their storage from step to step, so the tables are cached on the
+        tuple of their addresses: a steady-state call costs one pass that reads the addresses and
+        nothing else (no ctypes arrays are rebuilt, no tensor is examined again)."""
         if len(tensors) != len(self.layout):
             raise ValueError(f"expected {len(self.layout)} {what}s, got {len(tensors)}")
-        # one pass over the tensors (this runs every step, for every parameter); what exactly is
-        # wrong is worked out only when something is
-        live, addrs = [], []
+        key = tuple([0 if tensors[i] is None else tensors[i].data_ptr() for i in self._idx])
+        hit = self._addr_cache.get(what)
+        if hit is not None and hit[0] == key:
+            return hit[1]
+        # something moved (or this is the first call): look at every tensor; what exactly is wrong is
+        # worked out only when something is
+        live, addrs, staged = [], [], []
         numels, f32, dev_index = self.layout.numels, torch.float32, self._dev_index
         for i in self._idx:
             t = tensors[i]
             if t is None:
                 continue
-            if (t.numel() != numels[i] or t.dtype is not f32 or t.get_device() != dev_index
-                    or not t.is_contiguous()):
+            if t.numel() != numels[i] or t.dtype is not f32 or t.get_device() != dev_index:
                 self._refuse(tensors, what)
+            if not t.is_contiguous():
+                # e.g. a channels_last gradient: the kernels take flat memory, so it goes through a
+                # contiguous copy (and back, for an output)
+                with _stream_ctx(stream):
+                    tmp = t.contiguous()
+                staged.append((t, tmp))
+                t = tmp
             live.append(i)
             addrs.append(t.data_ptr())
-        key = tuple(live)
-        if key != self._live_key:
+        lkey = tuple(live)
+        if lkey != self._live_key:
             m = len(live)
-            self._live_key = key
+            self._live_key = lkey
             self._live_tabs = (
                 (ct.c_void_p * m)(*[self.grd_resi[i].data_ptr() for i in live]),
                 (ct.c_void_p * m)(*[self.grd_comp[i].data_ptr() for i in live]),
                 (ct.c_uint64 * m)(*[self.layout.numels[i] for i in live]),
                 (ct.c_uint64 * m)(*[self.layout.word_offset[i] for i in live]))
-        return (len(live), (ct.c_void_p * len(live))(*addrs)) + self._live_tabs
+        tabs = (len(live), (ct.c_void_p * len(live))(*addrs)) + self._live_tabs + (staged,)
+        # temporaries are new memory every call: only tables without them can be kept (one set for the
+        # gradients, one for the outputs, which may be other tensors)
+        self._addr_cache[what] = (key, tabs) if not staged else None
+        return tabs
 
     def _refuse(self, tensors, what):
         """Raise for the first tensor that does not fit: sizes first, then type, layout, device."""
@@ -167,8 +206,6 @@ class GradCompressor:
             t = tensors[i]
             if t.dtype != torch.float32 or not t.is_cuda:
                 raise TypeError(f"{what} {i}: expected a float32 GPU tensor, got {t.dtype} on {t.device}")
-            if not t.is_contiguous():
-                raise ValueError(f"{what} {i} must be contiguous")
             if t.device != self.resi.device:
                 raise ValueError(f"{what} {i} is on {t.device}, the buffers are on {self.resi.device}")
         raise AssertionError("unreachable: the quick check and the detailed one disagree")
@@ -178,11 +215,12 @@ class GradCompressor:
     def compress(self, grads, stream=None, sync=False):
         """Quantize every compressed parameter's gradient with error feedback.
 
-        `grads[i]` is parameter i's gradient (any shape, contiguous fp32 on the GPU), or None when
+        `grads[i]` is parameter i's gradient (any shape, fp32 on the GPU; one that is not contiguous,
+        such as a channels_last gradient, goes through a contiguous copy), or None when
         the parameter has no gradient this step (its residual and code words are left as they
         are); entries of uncompressed parameters are ignored.  One launch per 96 parameters.
         """
-        m, g_arr, r_arr, c_arr, n_arr, _ = self._tables(grads, "gradient")
+        m, g_arr, r_arr, c_arr, n_arr, _, _staged = self._tables(grads, "gradient", stream)
         if not m:
             return
         with _q._on_device(self.resi.device):
@@ -212,13 +250,16 @@ class GradCompressor:
         """outs[i] <- sum over ranks k = 0..kn-1 (in that order) of decode(recv[k] of parameter i),
         divided by kn when `average` (the `/ kn` of necklace/frmwrk/pytorch/ptprms.py:294).
         Entries that are None are skipped, as in `compress`."""
-        m, o_arr, _, _, n_arr, wo_arr = self._tables(outs, "output")
+        m, o_arr, _, _, n_arr, wo_arr, staged = self._tables(outs, "output", stream)
         if not m:
             return
         with _q._on_device(self.resi.device):
             _lib.check(_lib.lib().nklq_dequant_accumulate_multi_f32(
                 m, o_arr, n_arr, wo_arr, self._pl_arr, self.kn, self.thrd, 0,
                 float(self.kn) if average else 1.0, _nb.stream_handle(stream, self.resi.device)))
+            for t, tmp in staged:  # a non-contiguous output: the sums were written to its temporary
+                with _stream_ctx(stream):
+                    t.copy_(tmp)
         if sync:
             _sync(self.device, stream)
 
@@ -362,16 +403,65 @@ def grad_comp_state(grad_comp_cfg):
     """What has to go into the `state` dict handed to save_checkpoint
     (necklace/frmwrk/pytorch/callback.py:16-19) for the error feedback to survive a restart:
     the residual and the layout it belongs to.  Plain tensors and numbers only, so the file
-    loads with ``torch.load(..., weights_only=True)``."""
+    loads with ``torch.load(..., weights_only=True)``.
+
+    The bucket form lays its residuals out per bucket, and the buckets depend on which parameters
+    have a gradient; its state is therefore saved per PARAMETER (``param_resi``: position in the
+    optimizer's parameter list -> what that parameter is still owed, including the ones set aside
+    while a parameter sits a step out), which any later bucketing can take up again."""
     st = grad_comp_cfg["compressor"].state_dict()
-    return {"resi": st["resi"].detach().clone(), "thrd": float(st["thrd"]),
-            "numels": [int(n) for n in st["numels"]], "size_threshold": int(st["size_threshold"])}
+    out = {"resi": st["resi"].detach().clone(), "thrd": float(st["thrd"]),
+           "numels": [int(n) for n in st["numels"]], "size_threshold": int(st["size_threshold"])}
+    places = grad_comp_cfg.get("_places")
+    if grad_comp_cfg.get("_signature", ("",))[0] == "buckets" and places is not None:
+        gc = grad_comp_cfg["compressor"]
+        per = {int(pos): gc.grd_resi[bi][off:off + n].detach().clone() for pos, (bi, off, n) in places.items()}
+        for pos, r in grad_comp_cfg.get("_parked", {}).items():
+            per[int(pos)] = r.detach().clone()
+        out["form"] = "buckets"
+        out["param_resi"] = per
+    return out
 
 
 def load_grad_comp_state(grad_comp_cfg, state):
-    """Restore what `grad_comp_state` saved into a `grad_comp_cfg` built for the same parameters."""
-    grad_comp_cfg["compressor"].load_state_dict(state)
+    """Restore what `grad_comp_state` saved into a `grad_comp_cfg` for the same parameters.  When the
+    buffers are not laid out yet (a dict that has only been configured: the drop-ins below lay them
+    out on their first call), the state is kept in the dict and applied at that first call."""
+    gc = grad_comp_cfg.get("compressor")
     grad_comp_cfg["grad_comp_threshold"] = float(state["thrd"])
+    if gc is None or state.get("form") == "buckets":
+        grad_comp_cfg["_pending_state"] = state
+        if gc is not None:
+            gc.thrd = float(state["thrd"])
+        return
+    gc.load_state_dict(state)
+
+
+def _apply_pending_state(cfg, gc, places=None):
+    """Residuals loaded before the buffers existed: put them where the layout now has them."""
+    state = cfg.pop("_pending_state", None)
+    if state is None:
+        return
+    gc.thrd = float(state["thrd"])
+    per = state.get("param_resi")
+    if places is not None:  # bucket form: per-parameter residuals into their bucket slices
+        if per is None:
+            raise ValueError("the residual state was saved by the per-parameter form; it cannot be split over buckets")
+        parked = cfg.setdefault("_parked", {})
+        for pos, r in per.items():
+            where = places.get(int(pos))
+            if where is not None and where[2] == r.numel():
+                bi, off, n = where
+                gc.grd_resi[bi][off:off + n].copy_(r)
+            else:
+                parked[int(pos)] = r.to(gc.device).clone()
+    elif per is not None:   # saved by the bucket form, taken up by the per-parameter form
+        for pos, r in per.items():
+            pos = int(pos)
+            if pos < len(gc.grd_resi) and gc.grd_resi[pos] is not None and gc.grd_resi[pos].numel() == r.numel():
+                gc.grd_resi[pos].copy_(r)
+    else:
+        gc.load_state_dict(state)
 
 
 # --------------------------------------------------------------------------- ptprms call surface
@@ -420,7 +510,8 @@ def _small_fn(nc, cfg, root):
 
 def _take_buckets(tensors, limit_bytes):
     """Consecutive groups of tensors of at most `limit_bytes` each (a tensor larger than that is a
-    group of its own): the bucketing of ptprms.py:258 for tensors of one type."""
+    group of its own): the bucketing of ptprms.py:258 for tensors of one type (the callers have
+    checked that all are float32)."""
     buckets, cur, size = [], [], 0
     for t in tensors:
         b = t.numel() * t.element_size()
@@ -434,31 +525,72 @@ def _take_buckets(tensors, limit_bytes):
     return buckets
 
 
+def _rank_of(nc, cfg, kn):
+    """This worker's index among the kn: grad_comp_cfg['rank'], else nc.rank.  With several workers it
+    decides which receive slot holds the own payload and who decodes a reduce: a silent default of 0
+    on every worker would give wrong sums without any error."""
+    if "rank" in cfg:
+        return int(cfg["rank"])
+    r = getattr(nc, "rank", None)
+    if r is not None and not callable(r):
+        return int(r)
+    if kn > 1:
+        raise ValueError("grad_comp_cfg['rank'] (this worker's index, 0 .. kn-1) is required when kn > 1")
+    return 0
+
+
+def _check_fp32(grads):
+    """The compressed path packs fp32 gradients.  The reference buckets per tensor type
+    (_take_tensors, necklace/frmwrk/pytorch/ptprms.py:258) and all-reduces every type; here any other
+    type is refused before anything is launched (such gradients belong on the uncompressed path)."""
+    for i, g in enumerate(grads):
+        if g is not None and g.dtype != torch.float32:
+            raise TypeError(f"gradient {i} is {g.dtype}: the compressed exchange takes float32 gradients only")
+
+
 def _carry_residuals(old_gc, old_ids, new_gc, new_ids):
-    """Error feedback owed to a parameter survives a change of the layout."""
+    """Error feedback owed to a parameter survives a change of the layout: matched by parameter
+    identity when the old layout knows its parameters, by position otherwise (a layout that was
+    built or restored before the parameters were seen)."""
     if old_gc is None:
         return
-    where = {pid: i for i, pid in enumerate(old_ids)}
-    for j, pid in enumerate(new_ids):
-        i = where.get(pid)
+    if old_ids:
+        where = {pid: i for i, pid in enumerate(old_ids)}
+        pairs = [(where.get(pid), j) for j, pid in enumerate(new_ids)]
+    else:
+        pairs = [(j, j) for j in range(min(len(old_gc.grd_resi), len(new_gc.grd_resi)))]
+    for i, j in pairs:
         if i is not None and old_gc.grd_resi[i] is not None and new_gc.grd_resi[j] is not None \
                 and old_gc.grd_resi[i].numel() == new_gc.grd_resi[j].numel():
             new_gc.grd_resi[j].copy_(old_gc.grd_resi[i])
 
 
-def _cfg_for_params(params, kn, cfg):
+def _cfg_for_params(params, kn, cfg, nc=None):
     """Lay the buffers out over ALL parameters of the optimizer (a parameter without a gradient is
-    skipped per call); rebuilt, residuals carried over, when the optimizer's parameters change."""
+    skipped per call); rebuilt, residuals carried over, when the optimizer's parameters change.  A
+    compressor that is already in the dict and fits the parameters (from `init_grad_comp_cfg`,
+    possibly with residuals restored from a checkpoint) is taken as it is."""
     ids = [id(p) for p in params]
-    sig = ("params", tuple((i, p.numel()) for i, p in zip(ids, params)), kn)
+    numels = [p.numel() for p in params]
+    siz = int(cfg.get("grad_size_threshold", DEFAULT_SIZE_THRESHOLD))
+    sig = ("params", tuple(numels), kn, siz)
     if cfg.get("_signature") != sig:
         old_gc, old_ids = cfg.get("compressor"), cfg.get("_ids", [])
-        dev = params[0].device if params else torch.device("cuda")
-        built = init_grad_comp_cfg(params, kn, cfg, device=dev, rank=cfg.get("rank", 0))
-        _carry_residuals(old_gc if cfg.get("_signature", ("",))[0] == "params" else None, old_ids,
-                         built["compressor"], ids)
-        cfg.update(built)
+        was_params = cfg.get("_signature", ("params",))[0] == "params"
+        if old_gc is not None and "_signature" not in cfg and old_gc.kn == kn \
+                and old_gc.layout.numels == numels and old_gc.layout.size_threshold == siz:
+            gc = old_gc  # laid out beforehand for exactly these parameters
+            if "rank" in cfg and int(cfg["rank"]) != gc.rank:
+                raise ValueError(f"grad_comp_cfg['rank'] = {cfg['rank']}, its buffers were laid out for rank {gc.rank}")
+        else:
+            dev = params[0].device if params else torch.device("cuda")
+            built = init_grad_comp_cfg(params, kn, cfg, device=dev, rank=_rank_of(nc, cfg, kn))
+            gc = built["compressor"]
+            _carry_residuals(old_gc if was_params else None, old_ids, gc, ids)
+            cfg.update(built)
         cfg["_signature"], cfg["_ids"] = sig, ids
+    if "_pending_state" in cfg:  # residuals from a checkpoint, loaded before this layout existed
+        _apply_pending_state(cfg, cfg["compressor"])
     return cfg["compressor"]
 
 
@@ -484,8 +616,9 @@ def _reduce_small(small, kn, fn, average):
 
 
 def _reduce_params_form(nc, kn, root, params, cfg):
-    gc = _cfg_for_params(params, kn, cfg)
     grads = [p.grad.data if p.grad is not None else None for p in params]
+    _check_fp32(grads)
+    gc = _cfg_for_params(params, kn, cfg, nc)
     if all(g is None for g in grads):
         return
     average = root is None  # the reference's reduce leaves `/ kn` commented out (ptprms.py:385)
@@ -498,7 +631,7 @@ def _reduce_params_form(nc, kn, root, params, cfg):
 
 
 def _bucket_places(owners, buckets):
-    """{id of parameter: (bucket, offset, numel)} for a bucketing of the parameters' gradients."""
+    """{position of the parameter: (bucket, offset, numel)} for a bucketing of the parameters' gradients."""
     places, it = {}, iter(owners)
     for bi, bucket in enumerate(buckets):
         pos = 0
@@ -509,37 +642,42 @@ def _bucket_places(owners, buckets):
 
 
 def _reduce_buckets_form(nc, kn, root, params, cfg):
-    live = [p for p in params if p.grad is not None]
-    grads = [p.grad.data for p in live]
+    live = [(i, p) for i, p in enumerate(params) if p.grad is not None]
+    grads = [p.grad.data for _, p in live]
     if not grads:
         return
+    _check_fp32(grads)
     buckets = _take_buckets(grads, int(cfg.get("bucket_bytes", NCCL_REDUCE_BUCKET_BYTES)))
     sizes = [sum(g.numel() for g in b) for b in buckets]
     sig = ("buckets", tuple(tuple(g.numel() for g in b) for b in buckets), kn)
-    places = _bucket_places([id(p) for p in live], buckets)
+    # a parameter is known by its position in the optimizer's list: the same in every process and
+    # after a restart, which an id() is not
+    places = _bucket_places([i for i, _ in live], buckets)
     if cfg.get("_signature") != sig or cfg.get("_places") != places:
         old_gc, old_places = cfg.get("compressor"), cfg.get("_places")
         was_buckets = cfg.get("_signature", ("",))[0] == "buckets"
         sub = dict(cfg)
         sub["grad_size_threshold"] = 1  # a bucket is always packed
-        built = init_grad_comp_cfg(sizes, kn, sub, device=grads[0].device, rank=cfg.get("rank", 0))
+        built = init_grad_comp_cfg(sizes, kn, sub, device=grads[0].device, rank=_rank_of(nc, cfg, kn))
         if was_buckets and old_places:
             # the set of gradients changed: what a parameter is still owed moves to its new place;
             # a parameter that sits this step out has its residual set aside until it comes back
             parked = cfg.setdefault("_parked", {})
-            for pid, was in old_places.items():
-                if pid not in places:
-                    parked[pid] = old_gc.grd_resi[was[0]][was[1]:was[1] + was[2]].clone()
-            for pid, (bi, pos, n) in places.items():
-                was = old_places.get(pid)
+            for pos, was in old_places.items():
+                if pos not in places:
+                    parked[pos] = old_gc.grd_resi[was[0]][was[1]:was[1] + was[2]].clone()
+            for pos, (bi, off, n) in places.items():
+                was = old_places.get(pos)
                 if was is not None and was[2] == n:
-                    built["grd_resi"][bi][pos:pos + n].copy_(old_gc.grd_resi[was[0]][was[1]:was[1] + n])
-                elif was is None and pid in parked and parked[pid].numel() == n:
-                    built["grd_resi"][bi][pos:pos + n].copy_(parked.pop(pid))
+                    built["grd_resi"][bi][off:off + n].copy_(old_gc.grd_resi[was[0]][was[1]:was[1] + n])
+                elif was is None and pos in parked and parked[pos].numel() == n:
+                    built["grd_resi"][bi][off:off + n].copy_(parked.pop(pos))
         for key in ("grd_resi", "grd_recv", "grd_comp", "grd_cmps", "compressor"):
             cfg[key] = built[key]
         cfg["_signature"], cfg["_places"] = sig, places
         cfg["_flat"] = [torch.empty(n, dtype=torch.float32, device=grads[0].device) for n in sizes]
+    if "_pending_state" in cfg:  # residuals from a checkpoint, loaded before this layout existed (or over it)
+        _apply_pending_state(cfg, cfg["compressor"], places)
     gc, flats = cfg["compressor"], cfg["_flat"]
     for flat, bucket in zip(flats, buckets):  # grads_batch_coalesced, ptprms.py:262
         torch.cat([g.reshape(-1) for g in bucket], out=flat)
@@ -641,7 +779,8 @@ def opt_grads_fltn_do_nccl_reduce(nc, kn, root, d_arr_send, sz, grad_comp_cfg=No
         # first call (or another buffer length): lay the buffers out next to the flat gradient;
         # a residual from before belongs to another layout and does not carry over
         grad_comp_cfg.update(init_flat_grad_comp_cfg(sz, kn, grad_comp_cfg, device=d_arr_send.device,
-                                                     rank=grad_comp_cfg.get("rank", 0)))
+                                                     rank=_rank_of(nc, grad_comp_cfg, kn)))
         gc = grad_comp_cfg["compressor"]
+        _apply_pending_state(grad_comp_cfg, gc)
     opt_grads_fltn_do_compressed_reduce(kn, d_arr_send, sz, grad_comp_cfg, exchange=_exchange_of(nc),
                                         average=False, decode=gc.rank == root)

@@ -260,7 +260,7 @@ def test_model_form_gives_what_the_optimizer_form_gives():
     # the MXNet trainer's call shape: a dict of parameters, the receive buffers, nc, kn
     model_d, _, _, _ = _mlp_with_grads(seed=5)
     assert ptcomp.grads_do_nccl(dict(model_d.named_parameters()), None, TwoWorkersWithEqualData(), kn,
-                                grad_comp_cfg=dict(cfg_a)) is None
+                                grad_comp_cfg={"grad_comp_threshold": thrd, "grad_size_threshold": 1001}) is None
     torch.cuda.synchronize()
     for pa, pd in zip(model_a.parameters(), model_d.parameters()):
         assert torch.equal(pa.grad, pd.grad)
@@ -269,7 +269,7 @@ def test_model_form_gives_what_the_optimizer_form_gives():
     first = next(model_c.parameters())
     first.requires_grad_(False)
     stale = first.grad.clone()
-    cfg_c = dict(cfg_a)
+    cfg_c = {"grad_comp_threshold": thrd, "grad_size_threshold": 1001}
     ptcomp.grads_do_nccl_allreduce(TwoWorkersWithEqualData(), kn, model_c, None, grad_comp_cfg=cfg_c)
     torch.cuda.synchronize()
     assert torch.equal(first.grad, stale)
@@ -427,3 +427,101 @@ def test_sgd_with_compressed_gradients_still_learns():
         losses.append(float(loss.detach()))
     assert losses[-1] < 0.5 * losses[0], (losses[0], losses[-1])
     assert bool(torch.isfinite(cfg["compressor"].resi).all())
+
+
+def test_checkpoint_round_trip_through_the_drop_in_surface(tmp_path):
+    """Residual checkpointing as a trainer would use it (necklace/frmwrk/pytorch/callback.py:16-19):
+    step 1, save, "restart" (new model objects, a new grad_comp_cfg, load), step 2 through
+    opt_grads_do_nccl_allreduce must give exactly what two uninterrupted steps give — in both forms.
+    The layout step of the first call after the restart must not replace the restored residuals."""
+    for form in ("params", "buckets"):
+        thrd, kn = 1e-3, 2
+        base = {"grad_comp_threshold": thrd, "form": form, "bucket_bytes": 1 << 19}
+        # uninterrupted: two steps with one dict
+        model, opt, x, y = _mlp_with_grads(seed=11)
+        g1 = [p.grad.detach().clone() for p in model.parameters()]
+        cfg = dict(base)
+        ptcomp.opt_grads_do_nccl_allreduce(TwoWorkersWithEqualData(), kn, opt, None, grad_comp_cfg=cfg)
+        path = tmp_path / f"ckpt_{form}.pth.tar"
+        torch.save({"grad_comp": ptcomp.grad_comp_state(cfg)}, path)
+        g2 = [torch.randn_like(g) * 1e-3 for g in g1]   # the second step's gradients
+        for p, g in zip(model.parameters(), g2):
+            p.grad = g.clone()
+        ptcomp.opt_grads_do_nccl_allreduce(TwoWorkersWithEqualData(), kn, opt, None, grad_comp_cfg=cfg)
+        want = [p.grad.detach().clone() for p in model.parameters()]
+        # restart: other parameter objects, a dict that has only been configured, the state loaded into it
+        model2, opt2, _, _ = _mlp_with_grads(seed=11)
+        cfg2 = dict(base)
+        ptcomp.load_grad_comp_state(cfg2, torch.load(path, weights_only=True)["grad_comp"])
+        for p, g in zip(model2.parameters(), g2):
+            p.grad = g.clone()
+        ptcomp.opt_grads_do_nccl_allreduce(TwoWorkersWithEqualData(), kn, opt2, None, grad_comp_cfg=cfg2)
+        torch.cuda.synchronize()
+        for i, (p, w) in enumerate(zip(model2.parameters(), want)):
+            assert_bits_equal(p.grad.cpu().numpy(), w.cpu().numpy(), f"form {form}: parameter {i} after the restart")
+        assert torch.equal(cfg2["compressor"].resi.view(torch.int32), cfg["compressor"].resi.view(torch.int32)), form
+        assert float(cfg["compressor"].resi.abs().sum()) > 0
+        # without the state the second step differs (the test would pass trivially otherwise)
+        model3, opt3, _, _ = _mlp_with_grads(seed=11)
+        for p, g in zip(model3.parameters(), g2):
+            p.grad = g.clone()
+        ptcomp.opt_grads_do_nccl_allreduce(TwoWorkersWithEqualData(), kn, opt3, None, grad_comp_cfg=dict(base))
+        assert any(not torch.equal(p.grad, w) for p, w in zip(model3.parameters(), want))
+
+
+def test_a_gradient_that_is_not_contiguous_goes_through_a_copy():
+    """A channels_last gradient (what _flatten_dense_tensors accepts at ptprms.py:262) in the
+    per-parameter form: compressed from, and decoded into, a contiguous copy; the residual is laid
+    out in the gradient's logical (row-major) order."""
+    thrd, kn = 1e-3, 2
+    rng = np.random.default_rng(31)
+    w = torch.nn.Parameter(torch.zeros(16, 8, 5, 5, device="cuda"))
+    b = torch.nn.Parameter(torch.zeros(2000, device="cuda"))
+    gw = rng.normal(0, 1e-3, (16, 8, 5, 5)).astype(np.float32)
+    gb = rng.normal(0, 1e-3, 2000).astype(np.float32)
+    w.grad = dev(gw).contiguous(memory_format=torch.channels_last)
+    b.grad = dev(gb)
+    assert not w.grad.is_contiguous()
+    opt = torch.optim.SGD([w, b], lr=0.1)
+    cfg = {"grad_comp_threshold": thrd}
+    resid = [np.zeros(3200, np.float32), np.zeros(2000, np.float32)]
+    for step in range(2):   # twice: the tables are rebuilt every call while a temporary is involved
+        ptcomp.opt_grads_do_nccl_allreduce(TwoWorkersWithEqualData(), kn, opt, None, grad_comp_cfg=cfg)
+        torch.cuda.synchronize()
+        assert not w.grad.is_contiguous()
+        for i, (p, g) in enumerate(((w, gw), (b, gb))):
+            c, resid[i] = oracle.c.quantize(g.reshape(-1), thrd, R_in=resid[i])
+            want = (oracle.c.dequant_accumulate([c, c], g.size, thrd) / np.float32(kn)).astype(np.float32)
+            assert_bits_equal(p.grad.cpu().numpy().reshape(-1), want, f"step {step} parameter {i}")
+            assert_bits_equal(cfg["compressor"].grd_resi[i].cpu().numpy(), resid[i], f"step {step} residual {i}")
+        w.grad = dev(gw).contiguous(memory_format=torch.channels_last)
+        b.grad = dev(gb)
+
+
+def test_steady_state_calls_reuse_the_argument_tables():
+    """Gradients that keep their storage: the second call finds its tables by the gradients'
+    addresses; a gradient that moved is noticed and gives the right result."""
+    thrd = 1e-3
+    sizes = [3000, 10, 5000, 70000]
+    gc = ptcomp.GradCompressor(sizes, 1, thrd=thrd)
+    rng = np.random.default_rng(41)
+    hosts = [rng.normal(0, 1e-3, n).astype(np.float32) for n in sizes]
+    grads = [dev(h) for h in hosts]
+    gc.compress(grads, sync=True)
+    tabs = gc._addr_cache["gradient"][1]
+    for g, h in zip(grads, hosts):
+        g.copy_(torch.from_numpy(h))
+    gc.compress(grads, sync=True)
+    assert gc._addr_cache["gradient"][1] is tabs
+    resid = [None] * len(sizes)
+    for i, n in enumerate(sizes):
+        if gc.grd_cmps[i]:
+            _, r1 = oracle.c.quantize(hosts[i], thrd, R_in=np.zeros(n, np.float32))
+            c2, resid[i] = oracle.c.quantize(hosts[i], thrd, R_in=r1)
+            assert_words_equal(host_words(gc.grd_comp[i]), c2, f"parameter {i}")
+    moved = dev(hosts[2] * np.float32(2.0))     # parameter 2's gradient now lives elsewhere
+    grads[2] = moved
+    gc.compress(grads, sync=True)
+    assert gc._addr_cache["gradient"][1] is not tabs
+    c3, _ = oracle.c.quantize(hosts[2] * np.float32(2.0), thrd, R_in=resid[2])
+    assert_words_equal(host_words(gc.grd_comp[2]), c3, "the moved gradient")

@@ -80,7 +80,7 @@ def test_bucketing_follows_the_reference_rule():
 
 def test_layout_is_rebuilt_when_the_optimizer_changes_and_residuals_move_along():
     a, b = torch.nn.Parameter(torch.zeros(3000)), torch.nn.Parameter(torch.zeros(500))
-    cfg = {"grad_comp_threshold": 0.25, "grad_size_threshold": 1001}
+    cfg = {"grad_comp_threshold": 0.25, "grad_size_threshold": 1001, "rank": 0}
     gc1 = ptcomp._cfg_for_params([a, b], 2, cfg)
     assert gc1.grd_cmps == [True, False] and ptcomp._cfg_for_params([a, b], 2, cfg) is gc1  # kept while nothing changes
     gc1.grd_resi[0].copy_(torch.arange(3000, dtype=torch.float32))
@@ -118,3 +118,95 @@ def test_model_form_refuses_a_gradient_that_requires_grad():
     model.weight.grad = torch.zeros(3, 4)
     with pytest.raises(ValueError):  # the compressed path needs its configuration
         ptcomp.grads_do_nccl_allreduce(None, 1, model, None, grad_comp_cfg=None)
+
+
+def _params(*numels):
+    return [torch.nn.Parameter(torch.zeros(n)) for n in numels]
+
+
+def test_residuals_from_a_checkpoint_survive_the_first_drop_in_call():
+    """save -> new process -> init_grad_comp_cfg -> load -> first opt_*_do_nccl_* call: the layout step of
+    that call must take the restored compressor as it is, not build a zeroed one over it."""
+    params = _params(3000, 10, 5000)
+    cfg = ptcomp.init_grad_comp_cfg(params, 2, {"grad_comp_threshold": 0.25}, device="cpu", rank=1)
+    cfg["compressor"].resi.normal_()
+    state = ptcomp.grad_comp_state(cfg)
+    # a restart: same shapes, new parameter objects (other id()s), a fresh dict
+    params2 = _params(3000, 10, 5000)
+    cfg2 = ptcomp.init_grad_comp_cfg(params2, 2, {"grad_comp_threshold": 0.5}, device="cpu", rank=1)
+    ptcomp.load_grad_comp_state(cfg2, state)
+    want = state["resi"].clone()
+    gc = ptcomp._cfg_for_params(params2, 2, cfg2)
+    assert gc is cfg2["compressor"] and gc.rank == 1 and gc.thrd == 0.25
+    assert torch.equal(gc.resi, want) and float(want.abs().sum()) > 0
+    assert ptcomp._cfg_for_params(params2, 2, cfg2) is gc  # and it stays
+    # restored into a dict that has only been configured: kept until the first call lays the buffers out
+    cfg3 = {"grad_comp_threshold": 0.5, "rank": 1}
+    ptcomp.load_grad_comp_state(cfg3, state)
+    gc3 = ptcomp._cfg_for_params(_params(3000, 10, 5000), 2, cfg3)
+    assert torch.equal(gc3.resi, want) and gc3.thrd == 0.25 and "_pending_state" not in cfg3
+    # a state that belongs to other parameters is refused, not dropped
+    cfg4 = {"rank": 0}
+    ptcomp.load_grad_comp_state(cfg4, state)
+    with pytest.raises(ValueError):
+        ptcomp._cfg_for_params(_params(3000, 10, 5001), 2, cfg4)
+
+
+def test_bucket_state_is_kept_per_parameter_position():
+    """What the bucket form saves can be taken up by another bucketing (other bucket limits, a
+    parameter that sits out) and by the per-parameter form: it is keyed by the parameter's position."""
+    gc = ptcomp.GradCompressor([5000, 7000], kn=1, size_threshold=1, device="cpu")
+    gc.resi.normal_()
+    cfg = {"compressor": gc, "_signature": ("buckets", ((3000, 2000), (7000,)), 1),
+           "_places": {0: (0, 0, 3000), 2: (0, 3000, 2000), 3: (1, 0, 7000)},
+           "_parked": {1: torch.full((40,), 3.0)}}
+    state = ptcomp.grad_comp_state(cfg)
+    assert state["form"] == "buckets" and sorted(state["param_resi"]) == [0, 1, 2, 3]
+    assert torch.equal(state["param_resi"][2], gc.grd_resi[0][3000:5000])
+    assert torch.equal(state["param_resi"][1], torch.full((40,), 3.0))
+    # into one bucket of three of the parameters (position 2 has no gradient this step)
+    gc2 = ptcomp.GradCompressor([10040], kn=1, size_threshold=1, device="cpu")
+    cfg2 = {"_pending_state": state}
+    ptcomp._apply_pending_state(cfg2, gc2, {0: (0, 0, 3000), 1: (0, 3000, 40), 3: (0, 3040, 7000)})
+    assert torch.equal(gc2.grd_resi[0][:3000], state["param_resi"][0])
+    assert torch.equal(gc2.grd_resi[0][3000:3040], torch.full((40,), 3.0))
+    assert torch.equal(gc2.grd_resi[0][3040:], state["param_resi"][3])
+    assert torch.equal(cfg2["_parked"][2], state["param_resi"][2])   # set aside until it has a gradient again
+    # into the per-parameter form
+    gc3 = ptcomp.GradCompressor([3000, 40, 2000, 7000], kn=1, size_threshold=1001, device="cpu")
+    ptcomp._apply_pending_state({"_pending_state": state}, gc3)
+    assert torch.equal(gc3.grd_resi[0], state["param_resi"][0]) and gc3.grd_resi[1] is None
+    assert torch.equal(gc3.grd_resi[3], state["param_resi"][3])
+
+
+def test_rank_is_required_with_several_workers():
+    class Comm:
+        rank = 3
+    assert ptcomp._rank_of(None, {}, 1) == 0
+    assert ptcomp._rank_of(None, {"rank": 2}, 4) == 2
+    assert ptcomp._rank_of(Comm(), {}, 4) == 3          # taken from the communicator object
+    with pytest.raises(ValueError):
+        ptcomp._rank_of(None, {}, 2)
+    with pytest.raises(ValueError):
+        ptcomp._rank_of(lambda comp, recv: None, {}, 2)  # a bare exchange callable knows no rank
+    params = _params(3000)
+    with pytest.raises(ValueError):
+        ptcomp._cfg_for_params(params, 2, {})
+    with pytest.raises(ValueError):
+        ptcomp.opt_grads_fltn_do_nccl_reduce(None, 2, 0, torch.zeros(64), 64, grad_comp_cfg={})
+    cfg = ptcomp.init_grad_comp_cfg(params, 2, {"rank": 1}, device="cpu", rank=0)
+    with pytest.raises(ValueError):                      # the dict says 1, the buffers were laid out for 0
+        ptcomp._cfg_for_params(params, 2, cfg)
+
+
+def test_gradients_that_are_not_float32_are_refused_up_front():
+    """The reference buckets per tensor type (ptprms.py:258); the compressed path takes fp32 only and
+    says so before anything is laid out or launched."""
+    for form in ("params", "buckets"):
+        a, b = torch.nn.Parameter(torch.zeros(3000)), torch.nn.Parameter(torch.zeros(2000, dtype=torch.bfloat16))
+        a.grad, b.grad = torch.zeros(3000), torch.zeros(2000, dtype=torch.bfloat16)
+        opt = torch.optim.SGD([a, b], lr=0.1)
+        cfg = {"form": form}
+        with pytest.raises(TypeError, match="float32"):
+            ptcomp.opt_grads_do_nccl_allreduce(None, 1, opt, None, grad_comp_cfg=cfg)
+        assert "compressor" not in cfg
