@@ -647,8 +647,10 @@ def main():
         # the reference's own layout: (n, k) matrix, codes packed down the columns; wide and narrow,
         # rows on and off 128-byte lines
         res["matrix"] = {}
+        # (the last three: fewer than 8 bands of 16 rows, rows off 128-byte lines)
         for rows, cols in ((8192, 8192), (8191, 8191), (16384, 16383), (100000, 1000), (150_000, 401),
-                           (20_000_000, 3), (4_000_000, 17), (1_000_000, 65)):
+                           (20_000_000, 3), (4_000_000, 17), (1_000_000, 65),
+                           (16, 4_000_001), (100, 1_000_003), (144, 500_001)):
             tot = rows * cols
             A = g[:tot] if tot <= n else torch.randn(tot, device="cuda", generator=gen) * 1e-3
             R = torch.zeros(tot, device="cuda")

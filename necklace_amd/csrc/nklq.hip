@@ -28,7 +28,7 @@
 //     as two partial-line writes: views that start off a 128-byte line, and matrices whose rows
 //     do, get workgroup -> work maps that keep neighbours on one XCD, and the decodes move
 //     their grids onto lines (quant_flat_offline_kernel, deq_flat_shift_kernel, rows_tile_of);
-//   * the sum over K payloads (acc_flat_kernel), the matrix forms (quant_2d_rows_kernel for
+//   * the sum over K payloads (acc_flat_kernel), the matrix forms (quant_tiles_kernel for
 //     wide matrices, quant_bands_kernel for up to 384 columns) and the many-vectors form
 //     (quant_multi_kernel) are described at their kernels.
 //
@@ -57,6 +57,21 @@ typedef u32x4 u32x4_a4 __attribute__((aligned(4)));
 constexpr int kWave = 64;
 constexpr int kChunk = 256;          // elements per chunk: one dwordx4 per lane
 constexpr int kWordsPerChunk = 16;
+
+// Kernel arguments are fetched with scalar loads where the compiler first needs them; behind an early
+// exit that is a second round trip to memory before the kernel's first vector load can be issued, and
+// a short-lived workgroup lives about as long as its chain of round trips.  Naming the pointers here
+// makes the compiler fetch them at the top, together with the other arguments.
+template <typename P>
+__device__ __forceinline__ void fetch_argument_now(P ptr)
+{
+    asm volatile("" : : "s"(ptr));
+}
+template <typename... P>
+__device__ __forceinline__ void fetch_arguments_now(P... ptrs)
+{
+    (fetch_argument_now(ptrs), ...);
+}
 
 // ---------------------------------------------------------------- per element
 
@@ -542,85 +557,201 @@ __device__ __forceinline__ bool rows_tile_of(uint32_t b, uint32_t col_tiles, uin
     return *x < m;
 }
 
-// (Two or four 1 KiB pieces per wave and array, i.e. tiles of 512 or 1024 columns, measured 3-12 %
-// slower than one.)
-template <bool ADD, bool NT, bool ALIGNED>
-__global__ __launch_bounds__(kRowsBlock) void quant_2d_rows_kernel(
-    const float* g, const float* rin, float* rout, uint32_t* __restrict__ c, uint64_t n,
-    uint64_t k, uint32_t col_tiles, float t, uint32_t pinned)
+// ---- quantize by tiles of 16 rows x 128 columns (more than kBandsMaxColumns columns)
+//
+// A workgroup of 8 waves takes a tile; a wave moves two rows' pieces of 512 bytes, lane = 4
+// columns.  The 16 codes of a word come from 16 different lanes of 8 waves: every lane writes its 4
+// codes as 4 bytes into an image of the tile in LDS (row-major like the tile, no zeroing, no
+// atomics), and after ONE barrier 128 lanes gather the 16 bytes of their column into a word.
+// (Measured against the form it replaced, 16 waves x one row of 256 columns OR-ing codes into
+// zeroed LDS words between two barriers: 8192 x 8192 fused 0.81 -> 0.85 of the HBM peak,
+// 100000 x 1000 0.77 -> 0.81; 4 waves x 4 rows of 64 columns 0.76-0.80.)
+//
+// Rows that do not start on 128-byte lines make neighbouring tiles of a row share a line at their
+// common edge; written from two XCDs (two L2s) it reaches memory as two partial-line writes.
+//   * EDGES: the tiles of one band are given to ONE XCD (TileMap), where most shared lines merge:
+//     8191 x 8191 0.59 in plain order, 0.77 pinned.  Still 5 % more write requests than bytes / 64.
+//   * SHIFT: each row's window is moved left by the s = 0..31 elements the row's start lies past a
+//     line: columns [128 T - s, 128 T + 128 - s), so every store is whole lines.  The tile still owns
+//     the words of columns [128 T, 128 T + 128): the s elements its window misses at the right end are
+//     loaded a second time (8 lanes per row, one line, an L2 hit as the neighbour runs on the same
+//     XCD) for their codes only; their residual belongs to the neighbour.  That is a second reader
+//     of elements another workgroup updates, so this form is ONLY for calls whose residual output
+//     aliases neither input (the reference's own kernel, quantize.py:41-49, with R apart from A; the
+//     fused step with three buffers): in place, the neighbour may already have replaced r by r'.
+//     8191 x 8191 0.80, 16384 x 16383 0.81 against 0.77 / 0.76 with EDGES.
+
+// Workgroup -> (band x, column tile T).  Workgroups go to the 8 XCDs round-robin by id.  Plain order
+// (pinned = 0) when every row starts on a line.  Pinned: bands are dealt to the XCDs in groups of
+// 8, the tiles of a band run on one XCD in column order.  The last group may have fewer than 8
+// bands (all of them when the matrix has fewer than 128 rows): its bands are then cut into
+// 2^seg_shift segments of `seg_tiles` consecutive tiles, one XCD each, so that no XCD stays idle
+// (a 16 x 4,000,001 matrix would otherwise run on one XCD of eight).
+struct TileMap {
+    uint64_t inv_tiles;    // floor(2^64 / col_tiles) + 1
+    uint32_t col_tiles;
+    uint32_t full_blocks;  // workgroups of the full groups of 8 bands
+    uint32_t last_bands;   // bands of the last, smaller group (0: none)
+    uint64_t last_first;   // and the first of them
+    uint32_t seg_shift, seg_tiles;
+    uint32_t pinned;
+};
+
+__device__ __forceinline__ bool tile_of(const TileMap& tm, uint32_t b, uint64_t* x, uint32_t* T)
 {
-    constexpr int CQ = 1;        // 1 KiB pieces per wave and array
-    constexpr int W = 256 * CQ;  // columns per tile
-    __shared__ uint32_t words[W];
-    const int lane = threadIdx.x & (kWave - 1);
-    const uint32_t i = threadIdx.x >> 6;  // row inside the tile = code position inside the word
+    if (!tm.pinned) {
+        const uint32_t q = tm.col_tiles == 1 ? b : (uint32_t)__umul64hi((uint64_t)b, tm.inv_tiles);
+        *x = q;
+        *T = b - q * tm.col_tiles;
+        return true;
+    }
+    if (b < tm.full_blocks) {
+        const uint32_t e = b & 7u, j = b >> 3;
+        const uint32_t q = tm.col_tiles == 1 ? j : (uint32_t)__umul64hi((uint64_t)j, tm.inv_tiles);
+        *x = (uint64_t)q * 8 + e;
+        *T = j - q * tm.col_tiles;
+        return true;
+    }
+    const uint32_t bl = b - tm.full_blocks, e = bl & 7u, j = bl >> 3;
+    const uint32_t band = e >> tm.seg_shift, seg = e & ((1u << tm.seg_shift) - 1u);
+    *x = tm.last_first + band;
+    *T = seg * tm.seg_tiles + j;
+    return band < tm.last_bands && *T < tm.col_tiles;
+}
+
+// Elements [y, y + 4) of a row of k >= 4 elements; those outside the row read as 0.  ONE 16-byte load
+// for every lane, whole quad or not: a quad cut by an end of the row loads the four elements at that
+// end instead (address clamped into the row) and moves them into place.  (Loading the elements of a
+// cut quad one by one, in a branch of its own, made the compiler wait for the other lanes' loads
+// first: a second round trip to memory for every wave with a row end in it.)
+template <bool NT>
+__device__ __forceinline__ f32x4 ld4_row(const float* rowp, int64_t y, int64_t k)
+{
+    const int64_t yc = y < 0 ? 0 : (y + 4 > k ? k - 4 : y);
+    f32x4 w = ld4<false, NT>(rowp + yc);  // (dword alignment: the same global_load_dwordx4)
+    const int d = (int)(y - yc);          // -3 .. 3; element j of the quad is w[j + d]
+    if (d != 0) {
+        const float e[4] = {w.x, w.y, w.z, w.w};
+        float o[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            float v = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (i - j == d) v = e[i];   // (i - j ranges over -3 .. 3: at most one i per j matches)
+            o[j] = v;
+        }
+        w.x = o[0]; w.y = o[1]; w.z = o[2]; w.w = o[3];
+    }
+    return w;
+}
+
+// 4 codes as 4 bytes and the 4 residuals of a quad; the codes of elements outside the row are 0
+template <bool ADD>
+__device__ __forceinline__ uint32_t quant_quad(f32x4 va, f32x4 vr, float t, int64_t y, int64_t k, f32x4* o)
+{
+    f32x4 v = va;
+    if constexpr (ADD) v = v + vr;
+    float o0, o1, o2, o3;
+    uint32_t codes = quant_one(v.x, t, o0) | (quant_one(v.y, t, o1) << 8) | (quant_one(v.z, t, o2) << 16) |
+                     (quant_one(v.w, t, o3) << 24);
+    o->x = o0; o->y = o1; o->z = o2; o->w = o3;
+    if (!(y >= 0 && y + 4 <= k)) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (!(y + j >= 0 && y + j < k)) codes &= ~(0xFFu << (8 * j));
+    }
+    return codes;
+}
+
+// W columns per tile, Q quads per lane (4 W / Q threads): 128 x 1 when no line is shared between
+// tiles (rows on lines, or SHIFT), 256 x 1 with EDGES from 4096 columns (half as many shared lines:
+// 16384 x 16383 in place 0.74 with 128 columns, 0.78 with 256; but 150000 x 401 0.75 / 0.64) and for
+// matrices of a few bands.  More quads per lane (1024 columns per tile) measured no better anywhere.
+template <int W, int Q, bool ADD, bool NT, bool SHIFT>
+__global__ __launch_bounds__(4 * W / Q) void quant_tiles_kernel(
+    const float* g, const float* rin, float* rout, uint32_t* __restrict__ c, uint64_t n, uint64_t k, TileMap tm,
+    float t)
+{
+    constexpr int BLOCK = 4 * W / Q;           // 16 rows x (W / 4) quads / Q quads per lane
+    constexpr int TPR = W / 4 / Q;             // lanes per row
+    constexpr int ROWB = SHIFT ? W + 32 : W;   // image bytes per row: the window, and the 32 elements after it
+    static_assert(BLOCK == 16 * TPR && BLOCK <= 1024 && TPR >= 8, "tile geometry");
+    __shared__ __attribute__((aligned(16))) uint8_t image[16 * ROWB];
+    fetch_arguments_now(g, rin, rout, c);
     uint64_t x;
     uint32_t T;
-    if (!rows_tile_of(blockIdx.x, col_tiles, (n + 15) / 16, &x, &T, pinned)) return;
-    const uint64_t y0 = (uint64_t)T * W;
+    if (!tile_of(tm, blockIdx.x, &x, &T)) return;
+    if (x * 16 >= n) return;  // padding workgroups of the last group of 8 bands
+    const uint32_t i = threadIdx.x / TPR;  // row within the tile = code position within the word
+    const uint32_t l = threadIdx.x % TPR;  // lane within the row
     const uint64_t row = x * 16 + i;
-    int cnt[CQ];
-    uint64_t off[CQ];
-    float a[CQ][4], r[CQ][4];
+    const int64_t kk = (int64_t)k;
+    uint32_t codes[Q], codes_after = 0;
 #pragma unroll
-    for (int q = 0; q < CQ; ++q) {
-        const uint64_t y = y0 + 256 * q + (uint64_t)lane * 4;
-        // columns this lane owns in piece q: 4, or fewer at the right edge, or none
-        // (with ALIGNED, k is a multiple of 4: it is 4 or none)
-        cnt[q] = (row < n && y < k) ? ((ALIGNED || k - y >= 4) ? 4 : (int)(k - y)) : 0;
-        off[q] = row * k + y;
+    for (int q = 0; q < Q; ++q) codes[q] = 0;
+    if (row < n) {
+        const float* grow = g + row * k;
+        const float* rrow = rin + row * k;
+        float* orow = rout + row * k;
+        const int64_t s = SHIFT ? (int64_t)((reinterpret_cast<uintptr_t>(orow) >> 2) & 31u) : 0;
+        const int64_t y0 = (int64_t)T * W - s + 4 * l;      // this lane's first quad; the next ones 4 TPR columns on
+        const int64_t ya = y0 + W;                          // for the first lanes: the quad one window on
+        const bool on_after = SHIFT && 4 * (int64_t)l < s && ya < kk;
+        f32x4 va[Q], vr[Q], wa = {0.0f, 0.0f, 0.0f, 0.0f}, wr = wa;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) { a[q][j] = 0.0f; r[q][j] = 0.0f; }
-        if (cnt[q] == 4) {
-            const f32x4 va = ld4<ALIGNED, NT>(g + off[q]);
-            a[q][0] = va.x; a[q][1] = va.y; a[q][2] = va.z; a[q][3] = va.w;
-            if constexpr (ADD) {
-                const f32x4 vr = ld4<ALIGNED, NT>(rin + off[q]);
-                r[q][0] = vr.x; r[q][1] = vr.y; r[q][2] = vr.z; r[q][3] = vr.w;
+        for (int q = 0; q < Q; ++q) {
+            const int64_t y = y0 + 4 * TPR * q;
+            va[q] = wa;
+            vr[q] = wa;
+            if (y + 4 > 0 && y < kk) {
+                va[q] = ld4_row<NT>(grow, y, kk);
+                if constexpr (ADD) vr[q] = ld4_row<NT>(rrow, y, kk);
             }
-        } else {
+        }
+        if (on_after) {
+            wa = ld4_row<NT>(grow, ya, kk);
+            if constexpr (ADD) wr = ld4_row<NT>(rrow, ya, kk);
+        }
 #pragma unroll
-            for (int j = 0; j < 3; ++j) {
-                if (j < cnt[q]) {
-                    a[q][j] = g[off[q] + j];
-                    if constexpr (ADD) r[q][j] = rin[off[q] + j];
+        for (int q = 0; q < Q; ++q) {
+            const int64_t y = y0 + 4 * TPR * q;
+            if (y + 4 > 0 && y < kk) {
+                f32x4 o;
+                codes[q] = quant_quad<ADD>(va[q], vr[q], t, y, kk, &o);
+                if (y >= 0 && y + 4 <= kk) {
+                    st4<false, NT>(orow + y, o);  // (dword alignment: the same global_store_dwordx4)
+                } else {
+                    const float oe[4] = {o.x, o.y, o.z, o.w};
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        if (y + j >= 0 && y + j < kk) orow[y + j] = oe[j];
                 }
             }
         }
-    }
-    for (int wi = threadIdx.x; wi < W; wi += kRowsBlock) words[wi] = 0;
-    __syncthreads();
-    const uint32_t sh = 2 * i;
-#pragma unroll
-    for (int q = 0; q < CQ; ++q) {
-        if (cnt[q] > 0) {
-            float o[4];
-            uint32_t code[4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                float v = a[q][j];
-                if constexpr (ADD) v = v + r[q][j];
-                code[j] = quant_one(v, t, o[j]);
-            }
-            if (cnt[q] == 4) {
-                f32x4 vo;
-                vo.x = o[0]; vo.y = o[1]; vo.z = o[2]; vo.w = o[3];
-                st4<ALIGNED, NT>(rout + off[q], vo);
-            } else {
-#pragma unroll
-                for (int j = 0; j < 3; ++j)
-                    if (j < cnt[q]) rout[off[q] + j] = o[j];
-            }
-            // column 256 q + 4 lane + j lives at words[256 q + 64 j + lane]: consecutive lanes, consecutive banks
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-                if (j < cnt[q] && code[j]) atomicOr(&words[256 * q + 64 * j + lane], code[j] << sh);
+        if (on_after) {
+            f32x4 o;
+            codes_after = quant_quad<ADD>(wa, wr, t, ya, kk, &o);
         }
     }
+    // image[i][p] = code of column W T - s_i + p of row i
+#pragma unroll
+    for (int q = 0; q < Q; ++q) *reinterpret_cast<uint32_t*>(&image[i * ROWB + 4 * (l + TPR * q)]) = codes[q];
+    if (SHIFT && l < 8) *reinterpret_cast<uint32_t*>(&image[i * ROWB + W + 4 * l]) = codes_after;
     __syncthreads();
-    for (int wi = threadIdx.x; wi < W; wi += kRowsBlock) {
-        const int q = wi >> 8, cq = wi & 255;
-        if (y0 + wi < k) c[x * k + y0 + wi] = words[256 * q + 64 * (cq & 3) + (cq >> 2)];
+    for (uint32_t cc = threadIdx.x; cc < (uint32_t)W; cc += BLOCK) {
+        const uint64_t col = (uint64_t)T * W + cc;
+        if (col < k) {
+            uint32_t s = SHIFT ? (uint32_t)((reinterpret_cast<uintptr_t>(rout + x * 16 * k) >> 2) & 31u) : 0u;
+            const uint32_t k32 = (uint32_t)(k & 31u);
+            uint32_t word = 0;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                word |= (uint32_t)image[r * ROWB + cc + s] << (2 * r);
+                if constexpr (SHIFT) s = (s + k32) & 31u;  // the next row starts k elements on
+            }
+            c[x * k + col] = word;
+        }
     }
 }
 
@@ -633,13 +764,13 @@ __global__ __launch_bounds__(kRowsBlock) void quant_2d_rows_kernel(
 // read the tile's words (cache hits after the first).
 template <bool NT, bool SHIFT>
 __global__ __launch_bounds__(kRowsBlock) void deq_2d_rows_kernel(
-    float* out, const uint32_t* __restrict__ c, uint64_t n, uint64_t k, uint32_t col_tiles, float t)
+    float* out, const uint32_t* __restrict__ c, uint64_t n, uint64_t k, uint32_t col_tiles, float t, uint32_t pinned)
 {
     const int lane = threadIdx.x & (kWave - 1);
     const uint32_t i = threadIdx.x >> 6;
     uint64_t x;
     uint32_t T;
-    if (!rows_tile_of(blockIdx.x, col_tiles, (n + 15) / 16, &x, &T)) return;
+    if (!rows_tile_of(blockIdx.x, col_tiles, (n + 15) / 16, &x, &T, pinned)) return;
     const uint64_t row = x * 16 + i;
     if (row >= n) return;
     float* orow = out + row * k;
@@ -904,12 +1035,14 @@ constexpr uint64_t kStreamMaxColumns = 8192;
 template <bool NT>
 __global__ __launch_bounds__(256) void deq_stream_kernel(
     float* out, const uint32_t* __restrict__ c, uint64_t n, uint32_t k, uint32_t pieces, uint64_t inv_pieces,
-    uint32_t inv_k, float t)
+    uint32_t inv_k, float t, uint32_t pinned)
 {
-    const uint32_t xcd = blockIdx.x & 7u, j = blockIdx.x >> 3;
+    // pinned: bands dealt to the XCDs in groups of 8; else plain order (a matrix of a few bands: all XCDs busy,
+    // the words then come from the memory-side cache more than once)
+    const uint32_t xcd = pinned ? blockIdx.x & 7u : 0u, j = pinned ? blockIdx.x >> 3 : blockIdx.x;
     const uint32_t jb = (uint32_t)__umul64hi((uint64_t)j, inv_pieces);  // j / pieces
     const uint32_t q = j - jb * pieces;                                 // piece within the band
-    const uint64_t x = (uint64_t)jb * 8 + xcd;                          // band
+    const uint64_t x = pinned ? (uint64_t)jb * 8 + xcd : (uint64_t)jb;  // band
     if (x * 16 >= n) return;  // padding workgroups of the last group of 8 bands
     const uint32_t rows = n - x * 16 < 16 ? (uint32_t)(n - x * 16) : 16u;
     const int32_t blen = (int32_t)(rows * k);
@@ -1597,28 +1730,68 @@ int nklq_quantize_f32(const float* g, const float* r_in, float* r_out, uint32_t*
 #undef NKLQ_QB
         return launch_status();
     }
-    const bool al = (n_cols % 4 == 0) && aligned16(g) && aligned16(r_out) && (!add || aligned16(r_in));
-    // rows that do not all start on a 128-byte line: neighbouring tiles of a row share lines, keep them on one XCD
+    // tiles of 16 rows x 128 columns; which form (see quant_tiles_kernel):
     const bool on_lines = (n_cols % 32 == 0) && (reinterpret_cast<uintptr_t>(r_out) & 127u) == 0;
-    const uint32_t pinned = on_lines ? 0u : 1u;
-    const uint64_t col_tiles = (n_cols + 255) / 256;
-    const uint64_t m8 = pinned ? (m + 7) / 8 * 8 : m;  // pinned: word rows are dealt to the XCDs in groups of 8
-    if (col_tiles > 0x7FFFFFFFull || m8 > 0x7FFFFFFFull / col_tiles) return NKLQ_ERANGE;
-    const dim3 grid((uint32_t)(m8 * col_tiles)), block(kRowsBlock);
-#define NKLQ_Q2(ADD, NT, AL)                                                                        \
-    launch_kernel((quant_2d_rows_kernel<ADD, NT, AL>), grid, block, 0, s, g, r_in, r_out, c, n_rows, \
-                  n_cols, (uint32_t)col_tiles, thrd, pinned)
-    switch ((add ? 4 : 0) | (tk.nontemporal ? 2 : 0) | (al ? 1 : 0)) {
-        case 7: NKLQ_Q2(true, true, true); break;
-        case 6: NKLQ_Q2(true, true, false); break;
-        case 5: NKLQ_Q2(true, false, true); break;
-        case 4: NKLQ_Q2(true, false, false); break;
-        case 3: NKLQ_Q2(false, true, true); break;
-        case 2: NKLQ_Q2(false, true, false); break;
-        case 1: NKLQ_Q2(false, false, true); break;
-        default: NKLQ_Q2(false, false, false); break;
+    const uintptr_t o_lo = reinterpret_cast<uintptr_t>(r_out), o_hi = o_lo + 4 * total;
+    const auto clear_of = [&](const float* p) {
+        const uintptr_t lo = reinterpret_cast<uintptr_t>(p);
+        return lo + 4 * total <= o_lo || o_hi <= lo;
+    };
+    const bool shift = !on_lines && clear_of(g) && (!add || clear_of(r_in));  // r_out aliases no input
+    // tile width: 128 columns; 256 when tiles share lines and rows are long, and for matrices of a few bands
+    const bool few_bands = m < 32;
+    uint64_t tile_cols = few_bands || !(on_lines || shift || n_cols < 4096) ? 256 : 128;
+    TileMap tm = {};
+    const uint64_t col_tiles = ((shift ? n_cols + 31 : n_cols) + tile_cols - 1) / tile_cols;
+    if (col_tiles > 0x7FFFFFFFull) return NKLQ_ERANGE;
+    tm.col_tiles = (uint32_t)col_tiles;
+    tm.inv_tiles = col_tiles > 1 ? ~0ull / col_tiles + 1 : 0;  // floor(2^64 / col_tiles) + 1; with one tile per band it is not used
+    // Plain order when no line is shared between tiles, and for a few bands (there pinning leaves XCDs idle or
+    // with a short band: 100 x 1,000,003 in place 0.61 of the HBM peak in plain order, 0.56-0.58 pinned with the
+    // bands cut into segments; such shapes stay at 0.60-0.66 whatever the tile width, 128 to 1024 columns, and
+    // order: the 16 rows of a tile are megabytes apart)
+    tm.pinned = on_lines || few_bands ? 0u : 1u;
+    uint64_t blocks;
+    if (!tm.pinned) {
+        blocks = m * col_tiles;
+    } else {
+        const uint64_t full = (m / 8) * 8 * col_tiles;
+        tm.last_bands = (uint32_t)(m % 8);
+        tm.last_first = (m / 8) * 8;
+        blocks = full;
+        if (tm.last_bands) {
+            // 1 band -> 8 segments, 2 -> 4, 3 or 4 -> 2, more -> 1
+            tm.seg_shift = tm.last_bands == 1 ? 3u : (tm.last_bands == 2 ? 2u : (tm.last_bands <= 4 ? 1u : 0u));
+            tm.seg_tiles = (uint32_t)((col_tiles + (1u << tm.seg_shift) - 1) >> tm.seg_shift);
+            blocks += 8ull * tm.seg_tiles;
+        }
+        if (full > 0x7FFFFFFFull) return NKLQ_ERANGE;
+        tm.full_blocks = (uint32_t)full;
     }
-#undef NKLQ_Q2
+    if (blocks > 0x7FFFFFFFull) return NKLQ_ERANGE;
+    const dim3 grid((uint32_t)blocks);
+#define NKLQ_QT(W, Q, ADD, NT, SHIFT)                                                                      \
+    launch_kernel((quant_tiles_kernel<W, Q, ADD, NT, SHIFT>), grid, dim3(4 * W / Q), 0, s, g, r_in, r_out, c, \
+                  n_rows, n_cols, tm, thrd)
+#define NKLQ_QT_W(ADD, NT, SHIFT)                                  \
+    do {                                                           \
+        if (tile_cols == 128) NKLQ_QT(128, 1, ADD, NT, SHIFT);     \
+        else NKLQ_QT(256, 1, ADD, NT, SHIFT);                      \
+    } while (0)
+#define NKLQ_QT_FORM(ADD, NT)                  \
+    do {                                       \
+        if (shift) NKLQ_QT_W(ADD, NT, true);   \
+        else NKLQ_QT_W(ADD, NT, false);        \
+    } while (0)
+    switch ((add ? 2 : 0) | (tk.nontemporal ? 1 : 0)) {
+        case 3: NKLQ_QT_FORM(true, true); break;
+        case 2: NKLQ_QT_FORM(true, false); break;
+        case 1: NKLQ_QT_FORM(false, true); break;
+        default: NKLQ_QT_FORM(false, false); break;
+    }
+#undef NKLQ_QT_FORM
+#undef NKLQ_QT_W
+#undef NKLQ_QT
     return launch_status();
 }
 
@@ -1667,12 +1840,17 @@ int nklq_dequantize_f32(float* out, const uint32_t* c, uint64_t n_rows, uint64_t
     const bool plain = (n_cols % 32 == 0) && (reinterpret_cast<uintptr_t>(out) & 127u) == 0 && aligned16(c);
     if (n_cols > kStreamMaxColumns || (n_cols >= 4096 && plain)) {
         const uint64_t col_tiles = ((plain ? n_cols : n_cols + 31) + 255) / 256;
-        const uint64_t m8 = (m + 7) / 8 * 8;  // word rows are dealt to the XCDs in groups of 8
+        // No line is shared between tiles here and a tile's words are read by its own 16 waves: bands
+        // need not stay on one XCD.  They are still dealt to the XCDs in groups of 8 when there are many
+        // (each XCD sweeps one band: 0.93 against 0.91 at 16384 x 16383), in plain order when there are
+        // few (a 16 x 4,000,001 matrix would otherwise run on one XCD of eight)
+        const uint32_t pinned = m >= 32 ? 1u : 0u;
+        const uint64_t m8 = pinned ? (m + 7) / 8 * 8 : m;
         if (col_tiles > 0x7FFFFFFFull || m8 > 0x7FFFFFFFull / col_tiles) return NKLQ_ERANGE;
         const dim3 grid((uint32_t)(m8 * col_tiles)), block(kRowsBlock);
 #define NKLQ_D2(NT, SHIFT)                                                                        \
     launch_kernel((deq_2d_rows_kernel<NT, SHIFT>), grid, block, 0, s, out, c, n_rows, n_cols, \
-                       (uint32_t)col_tiles, thrd)
+                       (uint32_t)col_tiles, thrd, pinned)
         if (tk.nontemporal && plain) NKLQ_D2(true, false);
         else if (tk.nontemporal) NKLQ_D2(true, true);
         else if (plain) NKLQ_D2(false, false);
@@ -1682,17 +1860,18 @@ int nklq_dequantize_f32(float* out, const uint32_t* c, uint64_t n_rows, uint64_t
     }
     // everything else (97 .. 8192 columns): the band stream
     const uint64_t pieces = (16 * n_cols + 31 + 1023) / 1024;  // 4 KiB pieces of a band, on a grid that starts up to 31 elements before it
-    const uint64_t m8 = (m + 7) / 8 * 8;
+    const uint32_t pinned = m >= 32 ? 1u : 0u;
+    const uint64_t m8 = pinned ? (m + 7) / 8 * 8 : m;
     if (m8 > 0x7FFFFFFFull / pieces) return NKLQ_ERANGE;
     const uint32_t blocks = (uint32_t)(m8 * pieces);
     const uint64_t inv_pieces = ~0ull / pieces + 1;  // floor(2^64 / pieces) + 1 (pieces >= 2): exact quotients for j * pieces < 2^64
     const uint32_t inv_k = (uint32_t)(0x100000000ull / n_cols) + 1u;
     if (tk.nontemporal)
         launch_kernel((deq_stream_kernel<true>), dim3(blocks), dim3(256), 0, s, out, c, n_rows, (uint32_t)n_cols,
-                      (uint32_t)pieces, inv_pieces, inv_k, thrd);
+                      (uint32_t)pieces, inv_pieces, inv_k, thrd, pinned);
     else
         launch_kernel((deq_stream_kernel<false>), dim3(blocks), dim3(256), 0, s, out, c, n_rows, (uint32_t)n_cols,
-                      (uint32_t)pieces, inv_pieces, inv_k, thrd);
+                      (uint32_t)pieces, inv_pieces, inv_k, thrd, pinned);
     return launch_status();
 }
 

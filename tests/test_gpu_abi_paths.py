@@ -197,3 +197,52 @@ def test_compressor_with_more_than_sixteen_workers(kn, average):
         if average:
             want = (want / np.float32(kn)).astype(np.float32)
         assert_bits_equal(grads[i].cpu().numpy(), want, f"parameter {i} kn={kn} average={average}")
+
+
+# ------------------------------------------------------------------ few bands, many columns
+
+@pytest.mark.parametrize("n,k", [(16, 400_001), (7, 100_003), (100, 100_003), (144, 50_001), (33, 20_000), (129, 4_096),
+                                 (40, 12_345), (257, 1_000)])
+@pytest.mark.parametrize("in_place", [True, False])
+def test_wide_matrices_of_a_few_bands(n, k, in_place):
+    """Fewer than 8 bands of 16 rows, or a last group of fewer than 8: the tile map then cuts the
+    bands into segments so that every XCD has work; rows on and off 128-byte lines; the residual
+    updated in place (tiles that share lines at their edges) and written to a buffer of its own
+    (windows moved onto lines, the codes of each window's last columns computed by its neighbour too)."""
+    A, R0 = _data((n, k), n * 3 + k, 0.01)
+    if in_place:
+        L = _lib.lib()
+        g, r = dev(A), dev(R0)
+        m = (n + 15) // 16
+        c = torch.full((m, k), -1, dtype=torch.int32, device="cuda")
+        _lib.check(L.nklq_quantize_f32(g.data_ptr(), r.data_ptr(), r.data_ptr(), c.data_ptr(), n, k, 0.01, 1,
+                                       torch.cuda.current_stream().cuda_stream))
+        torch.cuda.synchronize()
+        want_c, want_r = oracle.c.quantize(A, 0.01, R_in=R0)
+        assert_words_equal(host_words(c), want_c, f"n={n} k={k}")
+        assert_bits_equal(r.cpu().numpy(), want_r, f"n={n} k={k}")
+        out = torch.full((n, k), 9.0, device="cuda")
+        _lib.check(L.nklq_dequantize_f32(out.data_ptr(), c.data_ptr(), n, k, 0.01, torch.cuda.current_stream().cuda_stream))
+        torch.cuda.synchronize()
+        assert_bits_equal(out.cpu().numpy(), oracle.c.dequantize(want_c, n, 0.01), f"decode n={n} k={k}")
+    else:
+        for og, oi, oo, oc in ((0, 0, 0, 0), (1, 2, 3, 1), (0, 0, 5, 0)):
+            _quantize_three_buffers(A, R0, 0.01, og, oi, oo, oc)
+
+
+@pytest.mark.parametrize("thrd", [0.0, -0.25, float("nan")])
+def test_tiles_with_thresholds_that_code_a_zero(thrd):
+    """With t <= 0 a value of 0 gets code 01: the lanes past the end of a row must not contribute codes."""
+    n, k = 37, 1_003
+    A, R0 = _data((n, k), 5, 0.01)
+    for og, oi, oo, oc in ((0, 0, 0, 0), (1, 2, 3, 1)):
+        _quantize_three_buffers(A, R0, thrd, og, oi, oo, oc)
+    g, r = dev(A), dev(R0)
+    c = torch.full(((n + 15) // 16, k), -1, dtype=torch.int32, device="cuda")
+    _lib.check(_lib.lib().nklq_quantize_f32(g.data_ptr(), r.data_ptr(), r.data_ptr(), c.data_ptr(), n, k, thrd, 1,
+                                            torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    with np.errstate(invalid="ignore"):
+        want_c, want_r = oracle.c.quantize(A, thrd, R_in=R0)
+    assert_words_equal(host_words(c), want_c, f"thrd={thrd}")
+    assert_bits_equal(r.cpu().numpy(), want_r, f"thrd={thrd}")
