@@ -386,6 +386,12 @@ def main():
         sys.exit(2)
     torch.cuda.set_device(0)
     L = _lib.lib()
+
+    def tuning():
+        """The measurement build of the same source (copy kernel, every launch geometry, interleaved sum)."""
+        hip_build.ensure_built(tuning=True)
+        return _lib.tuning_lib()
+
     n = args.elems
     gen = torch.Generator(device="cuda")
     gen.manual_seed(4)
@@ -600,20 +606,45 @@ def main():
             res["dequant_accumulate_by_payloads"][str(kp)] = {
                 "us": round(ev / 20 * 1e3, 1), "GBps": round(gb, 1), "frac_hbm_peak": frac(gb),
                 "payload_MB": round(4 * wl * kp / 1e6)}
-        del big, accl
+        del big
+        # The same 8 payloads' worth of words, the same bytes read and written, but the payloads
+        # alternate inside ONE array in runs of 2^s words: from 256 B runs (the 8 reads of a tile are one
+        # contiguous 2 KiB) to runs longer than a payload (8 streams far apart, the layout above).  If
+        # the number of distinct read streams were what slows the sum, short runs would be faster.
+        T = tuning()
+        nt = n - n % 1024
+        res["dequant_accumulate_by_interleave"] = {"payloads": K_PAYLOADS, "elements": nt}
+        top = max(6, (nt // 16 - 1).bit_length())
+        for s_log2 in (6, 8, 10, 12, 16, 20, top):
+            run = 1 << s_log2
+            runs = (nt // 16 + run - 1) // run
+            words = torch.randint(-2 ** 31, 2 ** 31 - 1, (runs * K_PAYLOADS * run,), dtype=torch.int32,
+                                  device="cuda", generator=gen)
+            f = lambda: _lib.check(T.nklq_tuning_sum_interleaved_f32(accl.data_ptr(), words.data_ptr(), K_PAYLOADS,
+                                                                     nt, s_log2, THRD, stream))
+            for _ in range(10):
+                f()
+            _, ev = time_region(torch, f, 20)
+            gb = (0.25 * K_PAYLOADS + 4) * nt / (ev / 20 * 1e-3) / 1e9
+            res["dequant_accumulate_by_interleave"][f"run_{4 * run}_bytes"] = {
+                "us": round(ev / 20 * 1e3, 1), "GBps": round(gb, 1), "frac_hbm_peak": frac(gb)}
+            del words
+        del accl
 
     if "geometry" in legs:
         # the launch knobs of nklq_tune on the three flat kernels at gradient size: the shipped defaults
         # against their neighbours (results never depend on them, only the time does)
         import ctypes as ct
-        default = [_lib.tune(i) for i in range(_lib.N_TUNE)]
+        Lg = tuning()     # the geometries other than the default exist in the measurement build only
+        tune = lambda i, v=-1: Lg.nklq_tune(i, v)
+        default = [tune(i) for i in range(_lib.N_TUNE)]
         wl = _lib.packed_words(n)
         pay = torch.randint(-2 ** 31, 2 ** 31 - 1, (K_PAYLOADS, wl), dtype=torch.int32, device="cuda", generator=gen)
         ptrg = (ct.c_void_p * K_PAYLOADS)(*[pay[p].data_ptr() for p in range(K_PAYLOADS)])
         kernels = {
-            "quantize": (lambda: _lib.check(L.nklq_quantize_f32(gp, rp, rp, cp, n, 1, THRD, 1, stream)), BYTES_QUANT),
-            "decode": (lambda: _lib.check(L.nklq_dequantize_f32(out.data_ptr(), cp, n, 1, THRD, stream)), BYTES_DEQUANT),
-            "sum8": (lambda: _lib.check(L.nklq_dequant_accumulate_f32(out.data_ptr(), ptrg, K_PAYLOADS, n, THRD, 0, stream)),
+            "quantize": (lambda: _lib.check(Lg.nklq_quantize_f32(gp, rp, rp, cp, n, 1, THRD, 1, stream)), BYTES_QUANT),
+            "decode": (lambda: _lib.check(Lg.nklq_dequantize_f32(out.data_ptr(), cp, n, 1, THRD, stream)), BYTES_DEQUANT),
+            "sum8": (lambda: _lib.check(Lg.nklq_dequant_accumulate_f32(out.data_ptr(), ptrg, K_PAYLOADS, n, THRD, 0, stream)),
                      0.25 * K_PAYLOADS + 4),
         }
         sweeps = {   # kernel -> [(label, {knob: value})]
@@ -630,9 +661,9 @@ def main():
             rows_ = {}
             for label, knobs in [("defaults", {})] + sweeps[name]:
                 for i, v in enumerate(default):
-                    _lib.tune(i, v)
+                    assert tune(i, v) >= 0
                 for kk, v in knobs.items():
-                    _lib.tune(kk, v)
+                    assert tune(kk, v) >= 0
                 for _ in range(5):
                     fn()
                 _, ev = time_region(torch, fn, 10)
@@ -640,7 +671,7 @@ def main():
                 rows_[label] = {"us": round(ev / 10 * 1e3, 1), "frac_hbm_peak": frac(gb)}
             res["launch_geometry"][name] = rows_
         for i, v in enumerate(default):
-            _lib.tune(i, v)
+            tune(i, v)
         del pay
 
     if "matrix" in legs:
@@ -717,8 +748,10 @@ def main():
         }
 
     if "copy" in legs:
+        T = tuning()   # the copy kernel is a measurement aid: it is not in the product library
+
         def cp():
-            _lib.check(L.nklq_copy_f32(out.data_ptr(), g.data_ptr(), n, stream))
+            _lib.check(T.nklq_copy_f32(out.data_ptr(), g.data_ptr(), n, stream))
 
         for _ in range(5):
             cp()

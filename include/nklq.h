@@ -151,22 +151,20 @@ int nklq_version(void);
  * (the sum over payloads only has its interleave knob).  Returns the previous
  * value, or NKLQ_ERANGE for an unknown knob or a value outside its set.
  * value < 0 only queries.  Safe to call while other threads launch.
+ *
+ * libnklq.so is built with ONE workgroup shape and the non-temporal forms
+ * only: there the first three knobs accept just the value in brackets.  The
+ * full sets belong to the measurement build of the same source
+ * (libnklq_tuning.so, include/nklq_tuning.h).
  */
-#define NKLQ_TUNE_CHUNKS_PER_WAVE 0      /* 256-element chunks per wave: 1, 2 or 4 */
-#define NKLQ_TUNE_WORKGROUP_SIZE 1       /* threads per workgroup: 64, 128, 256, 512 or 1024 */
-#define NKLQ_TUNE_NONTEMPORAL 2          /* non-temporal loads and stores of the fp32 streams: 0 or 1 */
+#define NKLQ_TUNE_CHUNKS_PER_WAVE 0      /* 256-element chunks per wave: [1], 2 or 4 */
+#define NKLQ_TUNE_WORKGROUP_SIZE 1       /* threads per workgroup: 64, 128, [256], 512 or 1024 */
+#define NKLQ_TUNE_NONTEMPORAL 2          /* non-temporal loads and stores of the fp32 streams: 0 or [1] */
 #define NKLQ_TUNE_XCD_INTERLEAVE_LOG2 3  /* quantize: neighbouring chunks are dealt to 2^v consecutive
                                             workgroups (which run on different XCDs): 0..6 */
 #define NKLQ_TUNE_XCD_INTERLEAVE_LOG2_DECODE 4  /* the same for dequantize */
 #define NKLQ_TUNE_XCD_INTERLEAVE_LOG2_ACCUMULATE 5  /* the same for the tiles (1024 elements) of the sum over payloads */
 int nklq_tune(int which, int value);
-
-/*
- * Measurement aid, not part of the quantizer: dst[i] = src[i] for n fp32
- * elements with the same 128-bit access pattern the quantizer uses.  Used to
- * calibrate HBM counters and to quote a copy bandwidth beside the kernels.
- */
-int nklq_copy_f32(float* dst, const float* src, uint64_t n, void* stream);
 
 #ifdef __cplusplus
 }

@@ -1,9 +1,14 @@
-"""Compiles csrc/nklq.hip into necklace_amd/libnklq.so for gfx950 (MI355X).
+"""Compiles csrc/nklq.hip for gfx950 (MI355X).
 
-    python -m necklace_amd.csrc.build
+    python -m necklace_amd.csrc.build            # necklace_amd/libnklq.so, the product library
+    python -m necklace_amd.csrc.build --tuning   # necklace_amd/libnklq_tuning.so as well
 
-hipcc cross-compiles without a GPU present.  The library is kept inside the
-package directory so that it is found next to the Python sources.
+The tuning library is the same source with -DNKLQ_TUNING_BUILD=1: every launch geometry nklq_tune
+can name, a copy kernel and the sum over interleaved payloads (include/nklq_tuning.h).  Only the
+geometry sweeps of bench.py and the parity tests that run every geometry load it.
+
+hipcc cross-compiles without a GPU present.  The libraries are kept inside the
+package directory so that they are found next to the Python sources.
 """
 import os
 import subprocess
@@ -13,6 +18,7 @@ CSRC = os.path.dirname(os.path.abspath(__file__))
 PKG = os.path.dirname(CSRC)
 ROOT = os.path.dirname(PKG)
 SO_PATH = os.path.join(PKG, "libnklq.so")
+TUNING_SO_PATH = os.path.join(PKG, "libnklq_tuning.so")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -25,9 +31,11 @@ FLAGS = [
 ]
 
 
-def build(verbose=False):
-    cmd = [HIPCC, *FLAGS, "-I", os.path.join(ROOT, "include"),
-           os.path.join(CSRC, "nklq.hip"), "-o", SO_PATH]
+def build(verbose=False, tuning=False):
+    """Compile the product library, or with tuning=True the measurement build of the same source."""
+    target = TUNING_SO_PATH if tuning else SO_PATH
+    cmd = [HIPCC, *FLAGS, *(["-DNKLQ_TUNING_BUILD=1"] if tuning else []), "-I", os.path.join(ROOT, "include"),
+           os.path.join(CSRC, "nklq.hip"), "-o", target]
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
@@ -38,15 +46,18 @@ def build(verbose=False):
         raise RuntimeError(f"hipcc failed ({res.returncode}):\n{out}")
     if verbose and out.strip():
         print(out)
-    return SO_PATH
+    return target
 
 
-def ensure_built():
+def ensure_built(tuning=False):
     """Build only when no library is there yet (a fresh checkout: the .so is not in version control)."""
-    if not os.path.exists(SO_PATH):
-        build()
-    return SO_PATH
+    target = TUNING_SO_PATH if tuning else SO_PATH
+    if not os.path.exists(target):
+        build(tuning=tuning)
+    return target
 
 
 if __name__ == "__main__":
     print(build(verbose="-q" not in sys.argv))
+    if "--tuning" in sys.argv:
+        print(build(verbose="-q" not in sys.argv, tuning=True))

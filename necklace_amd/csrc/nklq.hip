@@ -43,6 +43,9 @@
 #include <vector>
 
 #include "nklq.h"
+#if defined(NKLQ_TUNING_BUILD) && NKLQ_TUNING_BUILD
+#include "nklq_tuning.h"
+#endif
 
 namespace {
 
@@ -53,6 +56,19 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 // instructions need dword alignment only, so these still move 16 bytes per lane.
 typedef f32x4 f32x4_a4 __attribute__((aligned(4)));
 typedef u32x4 u32x4_a4 __attribute__((aligned(4)));
+
+// The product library carries one launch geometry (one chunk per wave, 256-thread workgroups) and the
+// non-temporal forms only.  Built with -DNKLQ_TUNING_BUILD=1 the same source also carries the other
+// geometries and the cached forms that nklq_tune can switch to, a plain copy kernel and the sum over
+// interleaved payloads (include/nklq_tuning.h): what the launch-geometry sweeps and the knob tests need.
+#ifndef NKLQ_TUNING_BUILD
+#define NKLQ_TUNING_BUILD 0
+#endif
+#if NKLQ_TUNING_BUILD
+#define NKLQ_NT(nt) (nt)
+#else
+#define NKLQ_NT(nt) true
+#endif
 
 constexpr int kWave = 64;
 constexpr int kChunk = 256;          // elements per chunk: one dwordx4 per lane
@@ -500,10 +516,14 @@ __device__ __forceinline__ void acc_tile(float* o, const PayloadPtrs& pl, int k_
     }
 }
 
-template <int K, bool ALIGNED, bool MIX>
+// RUNS (measurement builds only): the payloads are not k separate arrays but ONE array in which they
+// alternate in runs of 2^run_shift words (payload p's j-th run starts at word (j * k + p) << run_shift
+// of the array pl.p[0] points to; pl.p[p] = pl.p[0] + (p << run_shift)).  Same words, same bytes,
+// same arithmetic; only how far apart in memory the k reads of one tile are changes.
+template <int K, bool ALIGNED, bool MIX, bool RUNS = false>
 __global__ __launch_bounds__(kAccBlock) void acc_flat_kernel(
     float* acc, PayloadPtrs pl, int k_payloads, uint64_t n, uint64_t n_tiles, uint32_t has_tail,
-    uint32_t xs, float t, float th, int accumulate)
+    uint32_t xs, float t, float th, int accumulate, uint32_t run_shift)
 {
     __shared__ __attribute__((aligned(16))) float lds[kAccBlock / kWave][kAccLdsPerWave];
     const int lane = threadIdx.x & (kWave - 1);
@@ -517,7 +537,9 @@ __global__ __launch_bounds__(kAccBlock) void acc_flat_kernel(
     }
     const uint64_t tile = chunk_of<1, kAccBlock>(blockIdx.x, w, 0, xs);
     if (tile >= n_tiles) return;
-    acc_tile<K, ALIGNED, MIX, false>(acc + tile * kTile, pl, k_payloads, tile * (kTile / 16), t, th, accumulate,
+    uint64_t word0 = tile * (kTile / 16);
+    if constexpr (RUNS) word0 += ((word0 >> run_shift) * (uint64_t)((K > 0 ? K : k_payloads) - 1)) << run_shift;
+    acc_tile<K, ALIGNED, MIX, false>(acc + tile * kTile, pl, k_payloads, word0, t, th, accumulate,
                                      1.0f, 0.0f, lds[w], lane);
 }
 
@@ -1212,6 +1234,7 @@ __global__ __launch_bounds__(kAccBlock) void acc_multi_kernel(AccSegments seg, P
 
 // ---------------------------------------------------------------- copy (measurement aid)
 
+#if NKLQ_TUNING_BUILD
 template <int U, int BLOCK, bool NT>
 __global__ __launch_bounds__(BLOCK) void copy_kernel(float* dst, const float* src, uint64_t n,
                                                       uint64_t n_chunks, uint32_t has_tail,
@@ -1234,6 +1257,7 @@ __global__ __launch_bounds__(BLOCK) void copy_kernel(float* dst, const float* sr
     for (int j = 0; j < U; ++j)
         if (ch[j] < n_chunks) st4<true, NT>(dst + ch[j] * kChunk + lane * 4, a[j]);
 }
+#endif
 
 // ---------------------------------------------------------------- host side
 
@@ -1366,7 +1390,7 @@ int launch_quant_flat(const float* g, const float* rin, float* rout, uint32_t* c
     if (fg.blocks == 0) return NKLQ_ERANGE;
     const bool nt = tk.nontemporal != 0;
 #define NKLQ_Q(AL, ADD, NT)                                                                       \
-    launch_kernel((quant_flat_kernel<U, BLOCK, AL, ADD, NT>), dim3(fg.blocks), dim3(BLOCK), 0, \
+    launch_kernel((quant_flat_kernel<U, BLOCK, AL, ADD, NKLQ_NT(NT)>), dim3(fg.blocks), dim3(BLOCK), 0, \
                        s, g, rin, rout, c, n, fg.n_chunks, fg.has_tail, fg.xs, t)
     const int sel = (al ? 4 : 0) | (add ? 2 : 0) | (nt ? 1 : 0);
     switch (sel) {
@@ -1392,7 +1416,7 @@ int launch_deq_flat(float* out, const uint32_t* c, uint64_t n, float t, hipStrea
         launch_kernel((deq_flat_kernel<U, BLOCK, true>), dim3(fg.blocks), dim3(BLOCK), 0, s, out, c, n,
                       fg.n_chunks, fg.has_tail, fg.xs, t);
     else
-        launch_kernel((deq_flat_kernel<U, BLOCK, false>), dim3(fg.blocks), dim3(BLOCK), 0, s, out, c, n,
+        launch_kernel((deq_flat_kernel<U, BLOCK, NKLQ_NT(false)>), dim3(fg.blocks), dim3(BLOCK), 0, s, out, c, n,
                       fg.n_chunks, fg.has_tail, fg.xs, t);
     return launch_status();
 }
@@ -1454,13 +1478,14 @@ int launch_acc_flat(float* acc, const PayloadPtrs& pl, int k, uint64_t n, float 
     const uint32_t pad = n_tiles >= kAccThrottleTiles ? kAccThrottleLdsBytes : 0u;
 #define NKLQ_ACC(K, AL, MIX)                                                                        \
     launch_kernel((acc_flat_kernel<K, AL, MIX>), dim3(blocks), dim3(kAccBlock), pad, s, acc, pl, k, n, \
-                       n_tiles, has_tail, xs, t, th, accumulate)
+                       n_tiles, has_tail, xs, t, th, accumulate, 0u)
     NKLQ_ACC_DISPATCH(NKLQ_ACC, k, al, mix);
 #undef NKLQ_ACC
     return launch_status();
 }
 
 // Expands to the call of FN<U, BLOCK, ...> for the current knob values.
+#if NKLQ_TUNING_BUILD
 #define NKLQ_FOR_GEOMETRY(CALL)                                  \
     switch (tk.chunks_per_wave * 10000 + tk.block) {               \
         case 10064: return CALL(1, 64);                          \
@@ -1480,6 +1505,9 @@ int launch_acc_flat(float* acc, const PayloadPtrs& pl, int k, uint64_t n, float 
         case 41024: return CALL(4, 1024);                        \
         default: return NKLQ_ERANGE;                             \
     }
+#else
+#define NKLQ_FOR_GEOMETRY(CALL) return CALL(1, 256);
+#endif
 
 // Residual views that do not start on a 128-byte line take the kernel that keeps shared lines whole.
 int launch_quant_flat_offline(const float* g, const float* rin, float* rout, uint32_t* c, uint64_t n, float t,
@@ -1493,7 +1521,7 @@ int launch_quant_flat_offline(const float* g, const float* rin, float* rout, uin
     const dim3 grid((uint32_t)work + has_tail), block(256);
     const bool nt = tk.nontemporal != 0;
 #define NKLQ_QO(AL, ADD, NT) \
-    launch_kernel((quant_flat_offline_kernel<AL, ADD, NT>), grid, block, 0, s, g, rin, rout, c, n, n_chunks, has_tail, t)
+    launch_kernel((quant_flat_offline_kernel<AL, ADD, NKLQ_NT(NT)>), grid, block, 0, s, g, rin, rout, c, n, n_chunks, has_tail, t)
     switch ((al ? 4 : 0) | (add ? 2 : 0) | (nt ? 1 : 0)) {
         case 7: NKLQ_QO(true, true, true); break;
         case 6: NKLQ_QO(true, true, false); break;
@@ -1528,7 +1556,7 @@ int dispatch_deq_flat(float* out, const uint32_t* c, uint64_t n, float t, hipStr
         if (tk.nontemporal)
             launch_kernel((deq_flat_shift_kernel<true>), dim3((uint32_t)blocks), dim3(256), 0, s, out, c, n, n_chunks, d, t);
         else
-            launch_kernel((deq_flat_shift_kernel<false>), dim3((uint32_t)blocks), dim3(256), 0, s, out, c, n, n_chunks, d, t);
+            launch_kernel((deq_flat_shift_kernel<NKLQ_NT(false)>), dim3((uint32_t)blocks), dim3(256), 0, s, out, c, n, n_chunks, d, t);
         return launch_status();
     }
 #define NKLQ_CALL(U, B) launch_deq_flat<U, B>(out, c, n, t, s)
@@ -1536,6 +1564,7 @@ int dispatch_deq_flat(float* out, const uint32_t* c, uint64_t n, float t, hipStr
 #undef NKLQ_CALL
 }
 
+#if NKLQ_TUNING_BUILD
 template <int U, int BLOCK>
 int launch_copy(float* dst, const float* src, uint64_t n, hipStream_t s)
 {
@@ -1556,6 +1585,7 @@ int dispatch_copy(float* dst, const float* src, uint64_t n, hipStream_t s)
     NKLQ_FOR_GEOMETRY(NKLQ_CALL)
 #undef NKLQ_CALL
 }
+#endif
 
 // Workgroups for `total` wave items (chunks or tiles), 4 waves per workgroup, dealt over 2^xs.
 bool multi_grid(uint64_t total, uint32_t xs, uint32_t* blocks)
@@ -1575,7 +1605,7 @@ int launch_quant_multi(const QuantSegments& seg, bool al, bool add, float t, hip
     if (blocks == 0) return NKLQ_OK;
     const bool nt = tk.nontemporal != 0;
 #define NKLQ_QM(AL, ADD, NT) \
-    launch_kernel((quant_multi_kernel<AL, ADD, NT>), dim3(blocks), dim3(256), 0, s, seg, xs, t)
+    launch_kernel((quant_multi_kernel<AL, ADD, NKLQ_NT(NT)>), dim3(blocks), dim3(256), 0, s, seg, xs, t)
     switch ((al ? 4 : 0) | (add ? 2 : 0) | (nt ? 1 : 0)) {
         case 7: NKLQ_QM(true, true, true); break;
         case 6: NKLQ_QM(true, true, false); break;
@@ -1660,6 +1690,7 @@ int nklq_tune(int which, int value)
     if (which < 0 || which >= kKnobCount) return NKLQ_ERANGE;
     if (value < 0) return g_knobs[which].load(std::memory_order_relaxed);
     switch (which) {
+#if NKLQ_TUNING_BUILD
         case NKLQ_TUNE_CHUNKS_PER_WAVE:
             if (value != 1 && value != 2 && value != 4) return NKLQ_ERANGE;
             break;
@@ -1670,6 +1701,18 @@ int nklq_tune(int which, int value)
         case NKLQ_TUNE_NONTEMPORAL:
             value = value ? 1 : 0;
             break;
+#else
+        // the product library carries one form of each: only that value is accepted
+        case NKLQ_TUNE_CHUNKS_PER_WAVE:
+            if (value != 1) return NKLQ_ERANGE;
+            break;
+        case NKLQ_TUNE_WORKGROUP_SIZE:
+            if (value != 256) return NKLQ_ERANGE;
+            break;
+        case NKLQ_TUNE_NONTEMPORAL:
+            if (value != 1) return NKLQ_ERANGE;
+            break;
+#endif
         default:
             if (value > 6) return NKLQ_ERANGE;
             break;
@@ -1715,7 +1758,7 @@ int nklq_quantize_f32(const float* g, const float* r_in, float* r_out, uint32_t*
         const bool same = (reinterpret_cast<uintptr_t>(g) & 15u) == ph &&
                           (!add || (reinterpret_cast<uintptr_t>(r_in) & 15u) == ph);
 #define NKLQ_QB(ADD, NT, AL)                                                                          \
-    launch_kernel((quant_bands_kernel<ADD, NT, AL>), dim3(grid), dim3(kBandsBlock), 0, s, g, r_in, r_out, \
+    launch_kernel((quant_bands_kernel<ADD, NKLQ_NT(NT), AL>), dim3(grid), dim3(kBandsBlock), 0, s, g, r_in, r_out, \
                        c, n_rows, k32, per, inv, thrd)
         switch ((add ? 4 : 0) | (tk.nontemporal ? 2 : 0) | (same ? 1 : 0)) {
             case 7: NKLQ_QB(true, true, true); break;
@@ -1771,7 +1814,7 @@ int nklq_quantize_f32(const float* g, const float* r_in, float* r_out, uint32_t*
     if (blocks > 0x7FFFFFFFull) return NKLQ_ERANGE;
     const dim3 grid((uint32_t)blocks);
 #define NKLQ_QT(W, Q, ADD, NT, SHIFT)                                                                      \
-    launch_kernel((quant_tiles_kernel<W, Q, ADD, NT, SHIFT>), grid, dim3(4 * W / Q), 0, s, g, r_in, r_out, c, \
+    launch_kernel((quant_tiles_kernel<W, Q, ADD, NKLQ_NT(NT), SHIFT>), grid, dim3(4 * W / Q), 0, s, g, r_in, r_out, c, \
                   n_rows, n_cols, tm, thrd)
 #define NKLQ_QT_W(ADD, NT, SHIFT)                                  \
     do {                                                           \
@@ -1825,7 +1868,7 @@ int nklq_dequantize_f32(float* out, const uint32_t* c, uint64_t n_rows, uint64_t
         if (blocks > 0x7FFFFFFFull) return NKLQ_ERANGE;
         const uint32_t lds = 4u * (4u + 16u * per * k32);
 #define NKLQ_DB(NT, MIX)                                                                                      \
-    launch_kernel((deq_bands_kernel<NT, MIX>), dim3((uint32_t)blocks), dim3(kBandsBlock), lds, s, out, c, n_rows, \
+    launch_kernel((deq_bands_kernel<NKLQ_NT(NT), MIX>), dim3((uint32_t)blocks), dim3(kBandsBlock), lds, s, out, c, n_rows, \
                   k32, per, inv, thrd, th)
         if (tk.nontemporal && mix) NKLQ_DB(true, true);
         else if (tk.nontemporal) NKLQ_DB(true, false);
@@ -1849,7 +1892,7 @@ int nklq_dequantize_f32(float* out, const uint32_t* c, uint64_t n_rows, uint64_t
         if (col_tiles > 0x7FFFFFFFull || m8 > 0x7FFFFFFFull / col_tiles) return NKLQ_ERANGE;
         const dim3 grid((uint32_t)(m8 * col_tiles)), block(kRowsBlock);
 #define NKLQ_D2(NT, SHIFT)                                                                        \
-    launch_kernel((deq_2d_rows_kernel<NT, SHIFT>), grid, block, 0, s, out, c, n_rows, n_cols, \
+    launch_kernel((deq_2d_rows_kernel<NKLQ_NT(NT), SHIFT>), grid, block, 0, s, out, c, n_rows, n_cols, \
                        (uint32_t)col_tiles, thrd, pinned)
         if (tk.nontemporal && plain) NKLQ_D2(true, false);
         else if (tk.nontemporal) NKLQ_D2(true, true);
@@ -1870,7 +1913,7 @@ int nklq_dequantize_f32(float* out, const uint32_t* c, uint64_t n_rows, uint64_t
         launch_kernel((deq_stream_kernel<true>), dim3(blocks), dim3(256), 0, s, out, c, n_rows, (uint32_t)n_cols,
                       (uint32_t)pieces, inv_pieces, inv_k, thrd, pinned);
     else
-        launch_kernel((deq_stream_kernel<false>), dim3(blocks), dim3(256), 0, s, out, c, n_rows, (uint32_t)n_cols,
+        launch_kernel((deq_stream_kernel<NKLQ_NT(false)>), dim3(blocks), dim3(256), 0, s, out, c, n_rows, (uint32_t)n_cols,
                       (uint32_t)pieces, inv_pieces, inv_k, thrd, pinned);
     return launch_status();
 }
@@ -2046,6 +2089,7 @@ int nklq_dequant_accumulate_multi_f32(int count, float* const* acc, const uint64
     return NKLQ_OK;
 }
 
+#if NKLQ_TUNING_BUILD
 int nklq_copy_f32(float* dst, const float* src, uint64_t n, void* stream)
 {
     if (n == 0) return NKLQ_OK;
@@ -2058,5 +2102,42 @@ int nklq_copy_f32(float* dst, const float* src, uint64_t n, void* stream)
     snapshot_knobs();
     return dispatch_copy(dst, src, n, (hipStream_t)stream);
 }
+
+int nklq_tuning_sum_interleaved_f32(float* acc, const uint32_t* words, int k_payloads, uint64_t n,
+                                    int run_words_log2, float thrd, void* stream)
+{
+    if (k_payloads < 1 || k_payloads > NKLQ_MAX_PAYLOADS_PER_LAUNCH) return NKLQ_ERANGE;
+    if (run_words_log2 < 6 || run_words_log2 > 40 || n % kTile != 0) return NKLQ_ERANGE;
+    if (n == 0) return NKLQ_OK;
+    if (!acc || !words) return NKLQ_ENULL;
+    if (!aligned16(acc) || !aligned4(words)) return NKLQ_EALIGN;
+    const uint64_t run = 1ull << run_words_log2;
+    const uint64_t runs = (n / 16 + run - 1) / run;
+    if (runs > (UINT64_MAX >> run_words_log2) / (uint64_t)k_payloads) return NKLQ_ERANGE;
+    {
+        std::vector<Span> spans = {span_of(acc, 4 * n, true, 0),
+                                   span_of(words, 4 * runs * (uint64_t)k_payloads * run, false)};
+        if (spans_conflict(spans)) return NKLQ_EALIAS;
+    }
+    snapshot_knobs();
+    if (!mix_ok(thrd)) return NKLQ_ERANGE;
+    PayloadPtrs pl = {};
+    for (int p = 0; p < NKLQ_MAX_PAYLOADS_PER_LAUNCH; ++p) pl.p[p] = words + ((uint64_t)(p < k_payloads ? p : 0) << run_words_log2);
+    const uint64_t n_tiles = n / kTile;
+    const uint32_t xs = (uint32_t)tk.xcd_shift_acc;
+    const uint64_t per_group = (uint64_t)(kAccBlock / kWave) << xs;
+    const uint64_t work = ((n_tiles + per_group - 1) / per_group) << xs;
+    if (work > 0x7FFFFFFFull) return NKLQ_ERANGE;
+    const uint32_t pad = n_tiles >= kAccThrottleTiles ? kAccThrottleLdsBytes : 0u;
+    const float th = -0.5f * thrd;
+    hipStream_t s = (hipStream_t)stream;
+#define NKLQ_ACC_RUNS(K, AL, MIX)                                                                              \
+    launch_kernel((acc_flat_kernel<K, true, true, true>), dim3((uint32_t)work), dim3(kAccBlock), pad, s, acc, pl, \
+                  k_payloads, n, n_tiles, 0u, xs, thrd, th, 0, (uint32_t)run_words_log2)
+    NKLQ_ACC_DISPATCH(NKLQ_ACC_RUNS, k_payloads, true, true);
+#undef NKLQ_ACC_RUNS
+    return launch_status();
+}
+#endif
 
 }  // extern "C"

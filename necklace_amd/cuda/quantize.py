@@ -114,10 +114,11 @@ _fn_cache = {}
 
 
 def _fn(name):
-    """The bound ctypes function, looked up once."""
-    f = _fn_cache.get(name)
+    """The bound ctypes function of the library in use, looked up once per library."""
+    L = _lib.lib()
+    f = _fn_cache.get((L, name))
     if f is None:
-        f = _fn_cache[name] = getattr(_lib.lib(), name)
+        f = _fn_cache[(L, name)] = getattr(L, name)
     return f
 
 

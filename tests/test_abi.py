@@ -10,8 +10,8 @@ from conftest import ROOT
 from necklace_amd import _lib
 
 
-def _declared():
-    text = open(os.path.join(ROOT, "include", "nklq.h")).read()
+def _declared(header="nklq.h"):
+    text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(nklq_[a-z0-9_]+)\s*\(", text)))
 
@@ -23,6 +23,28 @@ def test_every_declared_symbol_is_exported_and_bound():
     for n in names:
         assert hasattr(L, n), f"{n} declared in nklq.h but not exported"
     assert sorted(_lib.SYMBOLS) == names
+    # what only serves measurements stays out of the product library
+    for n in _lib.TUNING_SYMBOLS:
+        assert not hasattr(L, n), f"{n} belongs to the measurement build only"
+
+
+def test_the_measurement_build_exports_both_headers():
+    T = _lib.tuning_lib()
+    extra = _declared("nklq_tuning.h")
+    assert sorted(_lib.TUNING_SYMBOLS) == extra
+    for n in _declared() + extra:
+        assert hasattr(T, n), f"{n} not exported by the measurement build"
+    assert T.nklq_version() == _lib.lib().nklq_version()
+    ok = 0x1000
+    assert T.nklq_copy_f32(None, None, 0, None) == 0
+    assert T.nklq_copy_f32(ok, ok + 2, 64, None) == -2
+    assert T.nklq_copy_f32(ok, ok + 16, 64, None) == -4
+    assert T.nklq_tuning_sum_interleaved_f32(None, None, 8, 0, 6, 0.5, None) == 0
+    assert T.nklq_tuning_sum_interleaved_f32(ok, ok + 0x100000, 8, 1000, 6, 0.5, None) == -3   # not whole tiles
+    assert T.nklq_tuning_sum_interleaved_f32(ok, ok + 0x100000, 8, 1024, 5, 0.5, None) == -3   # run below a tile's words
+    assert T.nklq_tuning_sum_interleaved_f32(ok, ok + 0x100000, 17, 1024, 6, 0.5, None) == -3
+    assert T.nklq_tuning_sum_interleaved_f32(ok, None, 8, 1024, 6, 0.5, None) == -1
+    assert T.nklq_tuning_sum_interleaved_f32(ok, ok + 1024, 8, 1024, 6, 0.5, None) == -4       # words inside acc
 
 
 def test_version_and_header_constants_agree():
@@ -110,19 +132,28 @@ def test_partial_overlaps_are_refused_without_a_launch():
     assert L.nklq_dequant_accumulate_multi_f32(2, accs, ns, woff, bases, 1, 0.5, 0, 1.0, None) == -4  # message over acc[1]
 
 
-def test_tune_knobs_round_trip():
-    for which, good, bad in ((0, (1, 2, 4), 3), (1, (64, 128, 256, 512, 1024), 96), (2, (0, 1), None),
-                             (3, (0, 1, 2, 3, 4, 5, 6), 7), (4, (0, 3, 6), 7), (5, (0, 3, 6), 7)):
+def _round_trip(cases):
+    for which, good, bad in cases:
         before = _lib.tune(which)
         for v in good:
             _lib.tune(which, v)
             assert _lib.tune(which) == v
-        if bad is not None:
+        for v in bad:
             with pytest.raises(ValueError):
-                _lib.tune(which, bad)
+                _lib.tune(which, v)
+        assert _lib.tune(which) == good[-1]
         _lib.tune(which, before)
     with pytest.raises(ValueError):
         _lib.tune(9, 1)
+
+
+def test_tune_knobs_round_trip():
+    """The product library has one workgroup shape: its first three knobs take their default only."""
+    interleave = ((3, (0, 1, 2, 3, 4, 5, 6), (7,)), (4, (0, 3, 6), (7,)), (5, (0, 3, 6), (7,)))
+    _round_trip(((0, (1,), (2, 3, 4)), (1, (256,), (64, 96, 1024)), (2, (1,), (0,))) + interleave)
+    with _lib.use_tuning_library():
+        _round_trip(((0, (1, 2, 4), (3,)), (1, (64, 128, 256, 512, 1024), (96,)), (2, (0, 1), ())) + interleave)
+    assert _lib.lib() is not _lib.tuning_lib()
 
 
 def test_missing_library_is_an_error_not_a_fallback(monkeypatch, tmp_path):

@@ -27,12 +27,18 @@ def _knobs():
 
 @pytest.fixture(params=_knobs(), ids=lambda k: f"u{k[0]}-wg{k[1]}-nt{k[2]}-x{k[3]}-xd{k[4]}-xa{k[5]}")
 def knobs(request):
-    old = [_lib.tune(i) for i in range(_lib.N_TUNE)]
-    for i, v in enumerate(request.param):
-        _lib.tune(i, v)
-    yield request.param
-    for i, v in enumerate(old):
-        _lib.tune(i, v)
+    """The default geometry runs on the product library, the others on the measurement build of the
+    same source (the only one that carries them)."""
+    if request.param == _knobs()[0]:
+        yield request.param
+        return
+    with _lib.use_tuning_library():
+        old = [_lib.tune(i) for i in range(_lib.N_TUNE)]
+        for i, v in enumerate(request.param):
+            _lib.tune(i, v)
+        yield request.param
+        for i, v in enumerate(old):
+            _lib.tune(i, v)
 
 
 def test_kat_vectors_on_gpu(kat):
@@ -420,7 +426,13 @@ def test_two_host_threads_on_two_streams():
 
 def test_one_thread_turns_the_knobs_while_another_launches():
     """The launch knobs are process-wide atomics and every call works from one snapshot of them:
-    a thread that keeps changing them must not disturb the results (or the launches) of another."""
+    a thread that keeps changing them must not disturb the results (or the launches) of another.
+    (On the measurement build: the product library has one workgroup shape.)"""
+    with _lib.use_tuning_library():
+        _turn_the_knobs_while_another_thread_launches()
+
+
+def _turn_the_knobs_while_another_thread_launches():
     import threading
     rng = np.random.default_rng(56)
     n = 1_000_000 + 77
