@@ -705,6 +705,23 @@ def main():
             res["matrix"][f"{rows}x{cols}"] = {"fused_us": round(ev / 30 * 1e3, 1), "fused_GBps": round(fq, 1),
                                                "fused_frac_hbm_peak": frac(fq), "decode_us": round(ev2 / 30 * 1e3, 1),
                                                "decode_GBps": round(fd, 1), "decode_frac_hbm_peak": frac(fd)}
+            if cols > 384 and cols % 32:
+                # rows off 128-byte lines: with the new residual in a buffer of its own (no in-place partner)
+                # the tiles move each row's window onto lines; in place they cannot (a neighbour would
+                # read elements another workgroup has already replaced)
+                R2 = torch.empty(tot, device="cuda")
+
+                def mq2():
+                    _lib.check(L.nklq_quantize_f32(A.data_ptr(), R.data_ptr(), R2.data_ptr(), C.data_ptr(),
+                                                   rows, cols, THRD, 1, stream))
+
+                for _ in range(5):
+                    mq2()
+                _, ev3 = time_region(torch, mq2, 30)
+                fo = BYTES_QUANT * tot / (ev3 / 30 * 1e-3) / 1e9
+                res["matrix"][f"{rows}x{cols}"].update({"fused_out_of_place_us": round(ev3 / 30 * 1e3, 1),
+                                                        "fused_out_of_place_frac_hbm_peak": frac(fo)})
+                del R2
             del A, R, C
 
     if "multi" in legs:

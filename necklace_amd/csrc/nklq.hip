@@ -1780,7 +1780,10 @@ int nklq_quantize_f32(const float* g, const float* r_in, float* r_out, uint32_t*
         const uintptr_t lo = reinterpret_cast<uintptr_t>(p);
         return lo + 4 * total <= o_lo || o_hi <= lo;
     };
-    const bool shift = !on_lines && clear_of(g) && (!add || clear_of(r_in));  // r_out aliases no input
+    // r_out aliases no input, and rows long enough for the re-read right fringe (up to 31 elements per tile and
+    // row) to pay: 16384 x 16383 537 -> 514 us, 8191 x 8191 132 -> 128 us, but 100000 x 1000 188 -> 191 us and
+    // 150000 x 401 125 -> 170 us
+    const bool shift = !on_lines && n_cols >= 4096 && clear_of(g) && (!add || clear_of(r_in));
     // tile width: 128 columns; 256 when tiles share lines and rows are long, and for matrices of a few bands
     const bool few_bands = m < 32;
     uint64_t tile_cols = few_bands || !(on_lines || shift || n_cols < 4096) ? 256 : 128;

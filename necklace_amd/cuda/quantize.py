@@ -17,7 +17,17 @@ can see, all deliberate:
   ``A.shape[0]`` (:29-31), which only works for square inputs;
 * extra keyword arguments: ``add_residual`` (error feedback: a = A + R before
   quantizing, R updated in place) and ``sync`` (the reference always blocks
-  until the stream is idle, :104; pass ``sync=False`` to stay asynchronous).
+  until the stream is idle, :104; pass ``sync=False`` to stay asynchronous);
+* contiguous tensors only.  The library's entry points take a base pointer and
+  (rows, columns) with no leading dimension, so a row-strided view (``M[:, :k]``
+  of a wider matrix, a transposed or channels_last tensor) raises ValueError
+  here instead of being read with the wrong stride; numba device arrays carry
+  their strides and the reference kernels would index such a view correctly.
+  necklace's own callers pass flattened gradients
+  (necklace/frmwrk/pytorch/ptprms.py:262,374), which
+  are contiguous; a caller that holds a strided view passes ``x.contiguous()``
+  and copies the residual back.  1-D slices of a flat buffer (``flat[a:b]``) are
+  contiguous and are taken at any element offset.
 """
 import ctypes as ct
 

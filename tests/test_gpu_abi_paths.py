@@ -93,7 +93,8 @@ def test_flat_fused_out_of_place(n, og, oi, oo, oc):
 
 
 @pytest.mark.parametrize("n,k", [(5000, 3), (403, 65), (50, 384), (16, 3), (47, 17),      # bands
-                                 (300, 385), (129, 1000), (40, 8191), (33, 1024), (100, 2048)])  # row tiles
+                                 (300, 385), (129, 1000), (40, 8191), (33, 1024), (100, 2048),
+                                 (520, 4099), (16 * 41, 4128)])                              # row tiles
 @pytest.mark.parametrize("og,oi,oo,oc", OFFSETS)
 def test_matrix_fused_out_of_place(n, k, og, oi, oo, oc):
     A, R0 = _data((n, k), n * 13 + k + og + 3 * oi + 7 * oo, 0.01)
