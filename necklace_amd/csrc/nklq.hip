@@ -1357,6 +1357,25 @@ bool spans_conflict(std::vector<Span>& v)
     return false;
 }
 
+// The overlap check of a many-vectors call sorts a few hundred ranges; its answer depends on the
+// addresses and sizes alone.  A training loop passes the same tables step after step, so each host
+// thread remembers the last set it has checked and found free of overlaps, and a call with exactly
+// that set again (compared value by value, not by a hash) skips the sort.
+struct CheckedTables {
+    std::vector<uint64_t> seen;
+    std::vector<uint64_t> now;
+    void begin() { now.clear(); }
+    void add(const void* table, size_t entries)
+    {
+        const uint64_t* p = static_cast<const uint64_t*>(table);  // tables of pointers or of uint64_t
+        now.insert(now.end(), p, p + entries);
+    }
+    void add(uint64_t v) { now.push_back(v); }
+    bool known() const { return now == seen; }
+    void remember() { seen.swap(now); }
+};
+static_assert(sizeof(void*) == sizeof(uint64_t), "pointer tables are compared as 64-bit words");
+
 struct FlatGrid {
     uint64_t n_chunks;
     uint32_t has_tail;
@@ -1970,7 +1989,13 @@ int nklq_quantize_multi_f32(int count, const float* const* g, float* const* r, u
         if (!aligned4(g[i]) || !aligned4(r[i]) || !aligned4(c[i])) return NKLQ_EALIGN;
         if (n[i] / kChunk + 1 > 0x7FFFFFFFull) return NKLQ_ERANGE;
     }
-    {
+    thread_local CheckedTables checked;
+    checked.begin();
+    checked.add(g, (size_t)count);
+    checked.add(r, (size_t)count);
+    checked.add(c, (size_t)count);
+    checked.add(n, (size_t)count);
+    if (!checked.known()) {
         std::vector<Span> spans;
         spans.reserve(3 * (size_t)count);
         for (int i = 0; i < count; ++i) {
@@ -1980,6 +2005,7 @@ int nklq_quantize_multi_f32(int count, const float* const* g, float* const* r, u
             spans.push_back(span_of(g[i], 4 * n[i], false, 2 * i));
         }
         if (spans_conflict(spans)) return NKLQ_EALIAS;
+        checked.remember();
     }
     snapshot_knobs();
     hipStream_t s = (hipStream_t)stream;
@@ -2032,7 +2058,14 @@ int nklq_dequant_accumulate_multi_f32(int count, float* const* acc, const uint64
         if (!aligned4(acc[i])) return NKLQ_EALIGN;
         if (n[i] / kTile + 1 > 0x7FFFFFFFull) return NKLQ_ERANGE;
     }
-    {
+    thread_local CheckedTables checked;
+    checked.begin();
+    checked.add(acc, (size_t)count);
+    checked.add(n, (size_t)count);
+    checked.add(word_offset, (size_t)count);
+    checked.add(payload_base, (size_t)k_payloads);
+    checked.add((uint64_t)count);  // (where the first three tables end)
+    if (!checked.known()) {
         // every payload is read between its lowest and highest word any vector uses
         uint64_t w_lo = UINT64_MAX, w_hi = 0;
         std::vector<Span> spans;
@@ -2048,6 +2081,7 @@ int nklq_dequant_accumulate_multi_f32(int count, float* const* acc, const uint64
             for (int p = 0; p < k_payloads; ++p)
                 spans.push_back(span_of(payload_base[p] + w_lo, 4 * (w_hi - w_lo), false));
         if (spans_conflict(spans)) return NKLQ_EALIAS;
+        checked.remember();
     }
     snapshot_knobs();
     hipStream_t s = (hipStream_t)stream;

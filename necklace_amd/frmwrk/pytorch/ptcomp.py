@@ -27,12 +27,15 @@ is an fp32 add before quantizing; the sum over ranks is a strict left-to-right
 fp32 sum in rank order (fp32 sums of {0, +t, -t} depend on the order).
 """
 import ctypes as ct
+import operator
 
 import torch
 
 from ... import _lib
 from ...cuda import nbutils as _nb
 from ...cuda import quantize as _q
+
+_data_ptr = torch.Tensor.data_ptr
 
 CMP_RATIO = _q.CMP_RATIO
 DEFAULT_SIZE_THRESHOLD = 1001  # grad_size_threshold default, necklace/trainer/tnopmx.py:137
@@ -139,6 +142,8 @@ class GradCompressor:
         # addresses is fixed for the life of the buffers (built on first use, per subset of
         # parameters that have a gradient)
         self._idx = [i for i, c in enumerate(self.grd_cmps) if c]
+        self._pick = (operator.itemgetter(*self._idx) if len(self._idx) > 1
+                      else (lambda seq, idx=tuple(self._idx): tuple(seq[i] for i in idx)))
         self._live_key, self._live_tabs = None, None
         self._addr_cache = {}
         # what Tensor.get_device() returns for tensors that live where the buffers do; host tensors
@@ -157,7 +162,10 @@ class GradCompressor:
         nothing else (no ctypes arrays are rebuilt, no tensor is examined again)."""
         if len(tensors) != len(self.layout):
             raise ValueError(f"expected {len(self.layout)} {what}s, got {len(tensors)}")
-        key = tuple([0 if tensors[i] is None else tensors[i].data_ptr() for i in self._idx])
+        try:
+            key = tuple(map(_data_ptr, self._pick(tensors)))
+        except TypeError:  # a parameter without a tensor this step
+            key = tuple([0 if tensors[i] is None else tensors[i].data_ptr() for i in self._idx])
         hit = self._addr_cache.get(what)
         if hit is not None and hit[0] == key:
             return hit[1]

@@ -247,3 +247,45 @@ def test_tiles_with_thresholds_that_code_a_zero(thrd):
         want_c, want_r = oracle.c.quantize(A, thrd, R_in=R0)
     assert_words_equal(host_words(c), want_c, f"thrd={thrd}")
     assert_bits_equal(r.cpu().numpy(), want_r, f"thrd={thrd}")
+
+
+# ------------------------------------------------------------------ the remembered overlap check
+
+def test_a_remembered_overlap_check_is_for_exactly_those_tables():
+    """The many-vectors calls skip their overlap check when the tables are the ones the thread's last
+    checked call had; any other table, also one that differs in a single address, is checked again."""
+    import ctypes as ct
+    L = _lib.lib()
+    vp, u64 = ct.c_void_p, ct.c_uint64
+    n = 4096
+    rng = np.random.default_rng(9)
+    g = [torch.from_numpy(rng.normal(0, 0.01, n).astype(np.float32)).cuda() for _ in range(2)]
+    r = [torch.zeros(n, device="cuda") for _ in range(2)]
+    c = [torch.zeros(n // 16, dtype=torch.int32, device="cuda") for _ in range(2)]
+    ns = (u64 * 2)(n, n)
+    tab = lambda ts: (vp * 2)(*[t.data_ptr() for t in ts])
+    good = (tab(g), tab(r), tab(c))
+    bad_c = (vp * 2)(c[0].data_ptr(), r[1].data_ptr() + 4 * n - 64)      # c[1] ends inside r[1]
+    stream = torch.cuda.current_stream().cuda_stream
+    for _ in range(3):
+        assert L.nklq_quantize_multi_f32(2, *good, ns, 0.01, 1, stream) == 0
+        assert L.nklq_quantize_multi_f32(2, good[0], good[1], bad_c, ns, 0.01, 1, stream) == -4
+    torch.cuda.synchronize()
+    for i in range(2):   # three error-feedback steps were launched, none of the refused calls wrote anything
+        want_r = np.zeros(n, np.float32)
+        for _ in range(3):
+            want_c, want_r = oracle.c.quantize(g[i].cpu().numpy(), 0.01, R_in=want_r)
+        assert_words_equal(host_words(c[i]), want_c, f"vector {i}")
+        assert_bits_equal(r[i].cpu().numpy(), want_r, f"vector {i}")
+    acc = [torch.empty(n, device="cuda") for _ in range(2)]
+    msg = torch.cat(c).contiguous()
+    woff = (u64 * 2)(0, n // 16)
+    bases = (vp * 1)(msg.data_ptr())
+    over = (vp * 2)(acc[0].data_ptr(), acc[0].data_ptr() + 4 * n - 4)    # acc[1] starts inside acc[0]
+    for _ in range(3):
+        assert L.nklq_dequant_accumulate_multi_f32(2, tab(acc), ns, woff, bases, 1, 0.01, 0, 1.0, stream) == 0
+        assert L.nklq_dequant_accumulate_multi_f32(2, over, ns, woff, bases, 1, 0.01, 0, 1.0, stream) == -4
+    torch.cuda.synchronize()
+    for i in range(2):
+        assert_bits_equal(acc[i].cpu().numpy(),
+                          oracle.c.dequantize(msg[i * (n // 16):(i + 1) * (n // 16)].cpu().numpy().view(np.uint32), n, 0.01))
