@@ -27,7 +27,7 @@
 //   * a cache line shared by two waves must be completed inside ONE XCD's L2 or it reaches memory
 //     as two partial-line writes: views that start off a 128-byte line, and matrices whose rows
 //     do, get workgroup -> work maps that keep neighbours on one XCD, and the decodes move
-//     their grids onto lines (quant_flat_offline_kernel, deq_flat_shift_kernel, rows_tile_of);
+//     their grids onto lines (quant_flat_offline_kernel, deq_flat_shift_kernel, tile_of);
 //   * the sum over K payloads (acc_flat_kernel), the matrix forms (quant_tiles_kernel for
 //     wide matrices, quant_bands_kernel for up to 384 columns) and the many-vectors form
 //     (quant_multi_kernel) are described at their kernels.
@@ -546,24 +546,22 @@ __global__ __launch_bounds__(kAccBlock) void acc_flat_kernel(
 // ---------------------------------------------------------------- matrix (n, k) kernels
 
 // Word (x, y) packs rows 16x .. 16x+15 of column y (quantize.py:35-51), so the 16 codes of a
-// word are k floats apart in memory.  A workgroup of 16 waves takes a tile of 16 rows x 256
-// columns: wave i moves row 16x+i of the tile with one dwordx4 per lane (1 KiB contiguous, like
-// a flat chunk), so neighbouring workgroups (on different XCDs) touch neighbouring 1 KiB pieces
-// of the same rows.  The 16 codes of a word come from 16 different waves: each wave ORs its
-// code, shifted to its bit position, into the tile's 256 words in LDS; after a barrier 256
-// threads store the 1 KiB of words.  When k is not a multiple of 4 (or a base is not 16-byte
-// aligned) rows start at any element: ALIGNED = false issues the same loads with dword
-// alignment, and the last 1-3 columns of a row are moved one by one.  Matrices of up to
-// kBandsMaxColumns columns take the band kernels further down instead.
+// word are k floats apart in memory: the 16 rows behind one row of words are a "band".  Which
+// kernel a matrix takes depends on its number of columns k:
+//   quantize  k <= kBandsMaxColumns: quant_bands_kernel (bands streamed as flat memory)
+//             wider: quant_tiles_kernel (tiles of 16 rows x 128 or 256 columns)
+//   decode    k <= 96: deq_bands_kernel (LDS image of whole bands)
+//             97 .. 8192: deq_stream_kernel (no LDS; 4 KiB pieces of a band)
+//             wider, or from 4096 with every row on a 128-byte line: deq_2d_rows_kernel (16 waves,
+//             wave i = row i of a tile of 16 rows x 256 columns, one dwordx4 per lane)
+// Rows may start at any element (k not a multiple of 4, bases only 4-byte aligned): the same
+// 16-byte requests are issued with dword alignment, and quads cut by a row end are masked.
 constexpr int kRowsBlock = 16 * kWave;  // 1024 threads
 
-// Workgroup -> tile (word row x, column tile T).  Workgroups go to the 8 XCDs round-robin by id; the
-// tiles of one word row are given to ONE XCD, in column order, and 8 neighbouring word rows run
-// side by side on the 8 XCDs (pinned = 1; pinned = 0 is the plain row-major order, used when every
-// row starts on a line).  When rows do not start on cache-line boundaries (k not a multiple
-// of 32) neighbouring tiles of a row share a line at their common edge: written from one XCD the
-// two halves merge in that XCD's L2 into a full-line write, written from two XCDs they reach memory
-// as two partial-line writes.  Returns false for the padding workgroups of the last group of rows.
+// Workgroup -> tile (band x, column tile T) of the tile decode.  Workgroups go to the 8 XCDs
+// round-robin by id; pinned = 1: the tiles of one band are given to ONE XCD, in column order, and 8
+// neighbouring bands run side by side on the 8 XCDs; pinned = 0: plain row-major order.  Returns
+// false for the padding workgroups of the last group of bands.
 __device__ __forceinline__ bool rows_tile_of(uint32_t b, uint32_t col_tiles, uint64_t m, uint64_t* x,
                                              uint32_t* T, uint32_t pinned = 1)
 {
@@ -591,8 +589,9 @@ __device__ __forceinline__ bool rows_tile_of(uint32_t b, uint32_t col_tiles, uin
 //
 // Rows that do not start on 128-byte lines make neighbouring tiles of a row share a line at their
 // common edge; written from two XCDs (two L2s) it reaches memory as two partial-line writes.
-//   * EDGES: the tiles of one band are given to ONE XCD (TileMap), where most shared lines merge:
-//     8191 x 8191 0.59 in plain order, 0.77 pinned.  Still 5 % more write requests than bytes / 64.
+//   * EDGES: the tiles of one band are given to ONE XCD (TileMap), so that a line both tiles read is
+//     fetched once: 8191 x 8191 0.59 in plain order, 0.77 pinned.  The two halves of a shared line
+//     are still written separately: 4-6 % more 64-byte write requests than the bytes need.
 //   * SHIFT: each row's window is moved left by the s = 0..31 elements the row's start lies past a
 //     line: columns [128 T - s, 128 T + 128 - s), so every store is whole lines.  The tile still owns
 //     the words of columns [128 T, 128 T + 128): the s elements its window misses at the right end are
@@ -601,7 +600,8 @@ __device__ __forceinline__ bool rows_tile_of(uint32_t b, uint32_t col_tiles, uin
 //     of elements another workgroup updates, so this form is ONLY for calls whose residual output
 //     aliases neither input (the reference's own kernel, quantize.py:41-49, with R apart from A; the
 //     fused step with three buffers): in place, the neighbour may already have replaced r by r'.
-//     8191 x 8191 0.80, 16384 x 16383 0.81 against 0.77 / 0.76 with EDGES.
+//     8191 x 8191 0.80, 16384 x 16383 0.81 against 0.77 / 0.76 with EDGES; write requests then equal
+//     the bytes.  Used from 4096 columns on: below, the re-read fringe costs more than it saves.
 
 // Workgroup -> (band x, column tile T).  Workgroups go to the 8 XCDs round-robin by id.  Plain order
 // (pinned = 0) when every row starts on a line.  Pinned: bands are dealt to the XCDs in groups of
