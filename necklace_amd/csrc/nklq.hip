@@ -606,22 +606,32 @@ __device__ __forceinline__ bool rows_tile_of(uint32_t b, uint32_t col_tiles, uin
 // Workgroup -> (band x, column tile T).  Workgroups go to the 8 XCDs round-robin by id.  Plain order
 // (pinned = 0) when every row starts on a line.  Pinned: bands are dealt to the XCDs in groups of
 // 8, the tiles of a band run on one XCD in column order.  The last group may have fewer than 8
-// bands (all of them when the matrix has fewer than 128 rows): its bands are then cut into
-// 2^seg_shift segments of `seg_tiles` consecutive tiles, one XCD each, so that no XCD stays idle
-// (a 16 x 4,000,001 matrix would otherwise run on one XCD of eight).
+// bands: its bands are then cut into 2^seg_shift segments of `seg_tiles` consecutive tiles, one XCD
+// each, so that no XCD stays idle.
+// Plain order with runs (pinned = 0, run_shift > 0), for matrices of a few bands with rows off
+// lines: tiles in row-major order, but every XCD takes 2^run_shift NEIGHBOURING tiles of each group
+// of 8 * 2^run_shift, so that most lines shared between tiles are fetched by one XCD only while all
+// XCDs still work on the same few megabytes (16 x 4,000,001 in place: 0.62 of the HBM peak in plain
+// order, 0.67 / 0.70 / 0.69 with runs of 2 / 4 / 8; with whole bands or long segments per XCD 0.15-0.58).
 struct TileMap {
     uint64_t inv_tiles;    // floor(2^64 / col_tiles) + 1
     uint32_t col_tiles;
-    uint32_t full_blocks;  // workgroups of the full groups of 8 bands
+    uint32_t full_blocks;  // pinned: workgroups of the full groups of 8 bands; runs: workgroups in whole groups
     uint32_t last_bands;   // bands of the last, smaller group (0: none)
     uint64_t last_first;   // and the first of them
     uint32_t seg_shift, seg_tiles;
     uint32_t pinned;
+    uint32_t run_shift;
 };
 
 __device__ __forceinline__ bool tile_of(const TileMap& tm, uint32_t b, uint64_t* x, uint32_t* T)
 {
     if (!tm.pinned) {
+        if (tm.run_shift && b < tm.full_blocks) {
+            // within its group of 8 << run_shift workgroups: XCD (b & 7) takes tiles (b & 7) << run_shift ...
+            const uint32_t group = 8u << tm.run_shift, o = b & (group - 1);
+            b = (b - o) + ((o & 7u) << tm.run_shift) + (o >> 3);
+        }
         const uint32_t q = tm.col_tiles == 1 ? b : (uint32_t)__umul64hi((uint64_t)b, tm.inv_tiles);
         *x = q;
         *T = b - q * tm.col_tiles;
@@ -1811,14 +1821,18 @@ int nklq_quantize_f32(const float* g, const float* r_in, float* r_out, uint32_t*
     if (col_tiles > 0x7FFFFFFFull) return NKLQ_ERANGE;
     tm.col_tiles = (uint32_t)col_tiles;
     tm.inv_tiles = col_tiles > 1 ? ~0ull / col_tiles + 1 : 0;  // floor(2^64 / col_tiles) + 1; with one tile per band it is not used
-    // Plain order when no line is shared between tiles, and for a few bands (there pinning leaves XCDs idle or
-    // with a short band: 100 x 1,000,003 in place 0.61 of the HBM peak in plain order, 0.56-0.58 pinned with the
-    // bands cut into segments; such shapes stay at 0.60-0.66 whatever the tile width, 128 to 1024 columns, and
-    // order: the 16 rows of a tile are megabytes apart)
+    // Plain order when no line is shared between tiles, and (with short runs per XCD, see TileMap) for a few
+    // bands: there pinning leaves XCDs idle or with a short band (100 x 1,000,003 in place 0.61 of the HBM peak in
+    // plain order, 0.56-0.58 pinned with the bands cut into segments, 0.70 with runs of 4; the tile width, 128 to
+    // 1024 columns, made no difference)
     tm.pinned = on_lines || few_bands ? 0u : 1u;
     uint64_t blocks;
     if (!tm.pinned) {
         blocks = m * col_tiles;
+        if (!on_lines) {  // (a few bands, rows off lines)
+            tm.run_shift = 2;
+            tm.full_blocks = (uint32_t)((blocks >> (3 + tm.run_shift) << (3 + tm.run_shift)) & 0x7FFFFFFFull);
+        }
     } else {
         const uint64_t full = (m / 8) * 8 * col_tiles;
         tm.last_bands = (uint32_t)(m % 8);
