@@ -697,9 +697,10 @@ __device__ __forceinline__ uint32_t quant_quad(f32x4 va, f32x4 vr, float t, int6
 }
 
 // W columns per tile, Q quads per lane (4 W / Q threads): 128 x 1 when no line is shared between
-// tiles (rows on lines, or SHIFT), 256 x 1 with EDGES from 4096 columns (half as many shared lines:
-// 16384 x 16383 in place 0.74 with 128 columns, 0.78 with 256; but 150000 x 401 0.75 / 0.64) and for
-// matrices of a few bands.  More quads per lane (1024 columns per tile) measured no better anywhere.
+// tiles (rows on lines, or SHIFT), 256 x 1 with EDGES and long rows (half as many shared lines:
+// 16384 x 16383 in place 0.74 with 128 columns, 0.78 with 256; but 150000 x 401 0.75 / 0.64; the
+// host side has the rule) and for matrices of a few bands.  More quads per lane (1024 columns per
+// tile) measured no better anywhere.
 template <int W, int Q, bool ADD, bool NT, bool SHIFT>
 __global__ __launch_bounds__(4 * W / Q) void quant_tiles_kernel(
     const float* g, const float* rin, float* rout, uint32_t* __restrict__ c, uint64_t n, uint64_t k, TileMap tm,
@@ -1813,9 +1814,13 @@ int nklq_quantize_f32(const float* g, const float* r_in, float* r_out, uint32_t*
     // row) to pay: 16384 x 16383 537 -> 514 us, 8191 x 8191 132 -> 128 us, but 100000 x 1000 188 -> 191 us and
     // 150000 x 401 125 -> 170 us
     const bool shift = !on_lines && n_cols >= 4096 && clear_of(g) && (!add || clear_of(r_in));
-    // tile width: 128 columns; 256 when tiles share lines and rows are long, and for matrices of a few bands
+    // tile width: 128 columns; 256 for matrices of a few bands and when tiles share lines and rows are long: from
+    // 4096 columns, and from 1000 when rows do not even start on 16-byte boundaries (every quad of 3 rows in 4 is
+    // then split over two 16-byte pieces: 60000 x 1023 0.68 -> 0.74, 30000 x 2047 0.75 -> 0.78; below 1000
+    // columns the narrow tile stays ahead, 120000 x 513 0.73 against 0.67)
     const bool few_bands = m < 32;
-    uint64_t tile_cols = few_bands || !(on_lines || shift || n_cols < 4096) ? 256 : 128;
+    const bool long_rows = n_cols >= 4096 || (n_cols % 4 != 0 && n_cols >= 1000);
+    uint64_t tile_cols = few_bands || (!on_lines && !shift && long_rows) ? 256 : 128;
     TileMap tm = {};
     const uint64_t col_tiles = ((shift ? n_cols + 31 : n_cols) + tile_cols - 1) / tile_cols;
     if (col_tiles > 0x7FFFFFFFull) return NKLQ_ERANGE;

@@ -187,7 +187,8 @@ def test_config5_hbm_sizing_chunked_error_feedback():
         assert torch.equal(g[lo:hi].view(torch.int32), dev(want).view(torch.int32)), f"sum of chunk at {lo}"
 
 
-@pytest.mark.parametrize("n,k", [(4099, 8191), (1_000_003, 17), (100_003, 384), (50_001, 385), (2_000_001, 3)])
+@pytest.mark.parametrize("n,k", [(4099, 8191), (1_000_003, 17), (100_003, 384), (50_001, 385), (2_000_001, 3),
+                                 (20_011, 1023), (9_001, 2047), (20_005, 1000)])
 def test_large_matrices_every_kernel_regime_against_the_oracle(n, k):
     """Tens of millions of elements per shape: many workgroups per XCD, padded grids (word rows in
     groups of 8, band ranges in runs), rows off 128-byte lines; fused step with a residual, then the
