@@ -188,7 +188,8 @@ def test_config5_hbm_sizing_chunked_error_feedback():
 
 
 @pytest.mark.parametrize("n,k", [(4099, 8191), (1_000_003, 17), (100_003, 384), (50_001, 385), (2_000_001, 3),
-                                 (20_011, 1023), (9_001, 2047), (20_005, 1000)])
+                                 (20_011, 1023), (9_001, 2047), (20_005, 1000),
+                                 (16, 4_000_001), (100, 1_000_003), (144, 500_001)])   # a few bands, at the benchmark's sizes
 def test_large_matrices_every_kernel_regime_against_the_oracle(n, k):
     """Tens of millions of elements per shape: many workgroups per XCD, padded grids (word rows in
     groups of 8, band ranges in runs), rows off 128-byte lines; fused step with a residual, then the
