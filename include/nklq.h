@@ -49,12 +49,17 @@ extern "C" {
  * Replaces the kernel cu_knl_matrix_quantize_e (necklace/cuda/quantize.py:16-51)
  * and its launch wrapper cu_fn_matrix_quantize_e (:96-115).
  *
- *   g      device, fp32 [n_rows, n_cols] row-major: the matrix A of the reference
+ *   g      device, fp32 [n_rows, n_cols] row-major and contiguous (row i starts
+ *          n_cols floats after row i-1: there is no leading dimension): the
+ *          matrix A of the reference
  *   r_in   device, fp32 same shape: residual carried from the previous step;
  *          read only when add_residual != 0 (may be NULL otherwise)
  *   r_out  device, fp32 same shape: the matrix R of the reference (every
  *          element is written).  May be the same pointer as r_in (in-place
  *          error feedback) or as g; any other overlap returns NKLQ_EALIAS.
+ *          (A matrix whose rows do not start on 128-byte lines is fastest
+ *          when r_out overlaps neither input: the kernel can then write
+ *          whole lines.)
  *   c      device, uint32 [ceil(n_rows/16), n_cols] row-major: the matrix C
  *          (every word is overwritten, whatever it held)
  *   thrd   the threshold; it crosses as C float, i.e. rounded to fp32 exactly
@@ -113,7 +118,9 @@ int nklq_dequant_accumulate_f32(float* acc, const uint32_t* const* payloads, int
  * gradients are a list of separate tensors, and the per-parameter lists grd_resi / grd_comp /
  * grd_recv that necklace's trainer keeps (necklace/trainer/tnopmx.py:140-149) are lists of
  * separate buffers.  All array arguments are HOST arrays of `count` entries, read during the
- * call only.  Vectors with n[i] == 0 are skipped.
+ * call only.  Vectors with n[i] == 0 are skipped.  A host thread that passes the same tables
+ * again (same addresses and sizes, as a training loop does) is not charged the overlap check
+ * a second time.
  *
  * nklq_quantize_multi_f32: for every i the flat quantize of g[i] (n[i] elements) into c[i]
  * (ceil(n[i]/16) words); the residual r[i] is updated in place when add_residual != 0
