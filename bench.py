@@ -50,9 +50,9 @@ def parse():
                     help="elements per launch (multiple of 16); 0 = the whole gradient in one launch. "
                          "The HBM-sizing workload is --elems 2800000000 --chunk 268435456")
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="CPU-baseline time budget; 0 skips it")
-    ap.add_argument("--legs", default="deq,acc,configs,wrapper,matrix,multi,copy,cpu",
-                    help="extra legs after the timed quantize steps: deq, acc, configs, wrapper, matrix, multi, "
-                         "copy, cpu, and (off by default) accsweep, geometry (comma list, '' = none)")
+    ap.add_argument("--legs", default="deq,coldcodes,acc,configs,wrapper,matrix,multi,copy,cpu",
+                    help="extra legs after the timed quantize steps: deq, coldcodes, acc, configs, wrapper, matrix, "
+                         "multi, copy, cpu, and (off by default) accsweep, geometry (comma list, '' = none)")
     return ap.parse_args()
 
 
@@ -494,7 +494,7 @@ def main():
     }
 
     legs = {x for x in args.legs.split(",") if x}
-    if legs & {"deq", "copy", "geometry"}:
+    if legs & {"deq", "coldcodes", "copy", "geometry"}:
         out = torch.empty(n, dtype=torch.float32, device="cuda")
     if "deq" in legs:
 
@@ -511,6 +511,34 @@ def main():
             "GBps": round(BYTES_DEQUANT * n / (deq_ms * 1e-3) / 1e9, 1),
             "frac_hbm_peak": round(BYTES_DEQUANT * n / (deq_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
         }
+
+    if "coldcodes" in legs:
+        # The decode loop above finds its 89 MB of code words in the 256 MB memory-side cache (they were read by
+        # the launch before; after an exchange they would have just been written).  Here 0.25 GB of other memory
+        # is read between the launches, so the words come from HBM: each launch timed on its own, median of 12,
+        # without and with the decode's prefetch workgroups (nklq_tune knob NKLQ_TUNE_DECODE_PREFETCH; left to
+        # itself the library switches them on from 2^30 elements, where the words cannot all be in that cache)
+        other = torch.ones(62_500_000, device="cuda")
+
+        def one_cold_decode():
+            other.sum()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            _lib.check(L.nklq_dequantize_f32(out.data_ptr(), c.data_ptr(), n, 1, THRD, stream))
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1)
+
+        res["dequant_code_words_from_hbm"] = {}
+        before = _lib.tune(_lib.TUNE_DECODE_PREFETCH)
+        for label, knob in (("without_prefetch", 2), ("with_prefetch", 1)):
+            _lib.tune(_lib.TUNE_DECODE_PREFETCH, knob)
+            ts = sorted([one_cold_decode() for _ in range(15)][3:])   # the first three are warm-up
+            ms = ts[len(ts) // 2]
+            res["dequant_code_words_from_hbm"][label] = {
+                "ms": round(ms, 4), "frac_hbm_peak": frac(BYTES_DEQUANT * n / (ms * 1e-3) / 1e9)}
+        _lib.tune(_lib.TUNE_DECODE_PREFETCH, before)
+        del other
 
     if "acc" in legs:
         # receive side at bucket size: 8 payloads (local + 7 synthetic peers, P(0) = 0.9) into one buffer

@@ -171,6 +171,12 @@ int nklq_version(void);
                                             workgroups (which run on different XCDs): 0..6 */
 #define NKLQ_TUNE_XCD_INTERLEAVE_LOG2_DECODE 4  /* the same for dequantize */
 #define NKLQ_TUNE_XCD_INTERLEAVE_LOG2_ACCUMULATE 5  /* the same for the tiles (1024 elements) of the sum over payloads */
+#define NKLQ_TUNE_DECODE_PREFETCH 6      /* flat dequantize: extra workgroups read the code words ahead of the
+                                            decoding ones.  Pays when the words come from HBM (0.6 -> 0.88 of
+                                            the HBM peak), costs 6 % when they are in the 256 MB memory-side
+                                            cache anyway (just written or read).  0: only for vectors whose
+                                            words exceed that cache (2^30 elements and more); 1: always;
+                                            2: never */
 int nklq_tune(int which, int value);
 
 #ifdef __cplusplus

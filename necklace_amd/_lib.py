@@ -121,7 +121,8 @@ def packed_words(n_rows, n_cols=1):
 
 TUNE_CHUNKS_PER_WAVE, TUNE_WORKGROUP_SIZE, TUNE_NONTEMPORAL = 0, 1, 2
 TUNE_XCD_INTERLEAVE_LOG2, TUNE_XCD_INTERLEAVE_LOG2_DECODE, TUNE_XCD_INTERLEAVE_LOG2_ACCUMULATE = 3, 4, 5
-N_TUNE = 6
+TUNE_DECODE_PREFETCH = 6
+N_TUNE = 7
 
 
 def tune(which, value=-1):

@@ -310,10 +310,21 @@ __global__ __launch_bounds__(256) void quant_flat_offline_kernel(
 // with ordinary (cached) loads: two chunks share a 128 B line, and non-temporal loads of half
 // lines measure 20-35 % slower here.  The target starts on a 128-byte line (any other start takes
 // deq_flat_shift_kernel), so every store is a whole aligned 16 bytes.
+//
+// A workgroup here lives about as long as its one read of code words takes, and the chip holds a
+// fixed number of them: when the words come from HBM instead of the memory-side cache (they were
+// not written or read just before, or there are more of them than the cache holds) the read takes
+// 2-3 times as long and the whole decode runs at 0.6 of the HBM peak instead of 0.95.  pf_lead > 0
+// (xs = 0 only) adds 8 prefetch workgroups, one per XCD, behind every 256 working ones: each reads
+// one word of every 128-byte line of code words that the workgroups pf_lead blocks of 256 further
+// on will need, which brings the lines into the memory-side cache: 0.88 with words from HBM.  The
+// second trip of the words over the fabric costs their share of the bytes, 6 %, when they were in the
+// cache anyway (0.89 against 0.95), so the host side asks for it only where they cannot be.
+constexpr uint32_t kPrefetchBlock = 256;  // working workgroups per block; 8 prefetching ones follow
 template <int U, int BLOCK, bool NT>
 __global__ __launch_bounds__(BLOCK) void deq_flat_kernel(
     float* out, const uint32_t* __restrict__ c, uint64_t n, uint64_t n_chunks, uint32_t has_tail,
-    uint32_t xs, float t)
+    uint32_t xs, float t, uint32_t pf_lead)
 {
     if (has_tail && blockIdx.x == gridDim.x - 1) {
         // tail: one element per lane, bounds-checked
@@ -324,12 +335,29 @@ __global__ __launch_bounds__(BLOCK) void deq_flat_kernel(
         }
         return;
     }
+    uint32_t b = blockIdx.x;
+    if (pf_lead) {
+        // working workgroup p of the vector stays on XCD p % 8, as without prefetching
+        const uint32_t q = b / (kPrefetchBlock + 8), r = b - q * (kPrefetchBlock + 8);
+        if (r >= kPrefetchBlock) {
+            constexpr uint32_t words = (kPrefetchBlock / 8) * (BLOCK / kWave) * U * kWordsPerChunk;  // an eighth of a block's
+            const uint64_t first = ((uint64_t)(q + pf_lead) * 8 + (r - kPrefetchBlock)) * words;
+            uint32_t bits = 0;
+            for (uint32_t i = threadIdx.x; i < words / 32; i += BLOCK) {
+                const uint64_t wi = first + 32ull * i;
+                if (wi < n_chunks * kWordsPerChunk) bits ^= c[wi];
+            }
+            asm volatile("" : : "v"(bits));  // (the loads have to be issued and waited for; their values are not used)
+            return;
+        }
+        b = q * kPrefetchBlock + r;
+    }
     const int lane = threadIdx.x & (kWave - 1);
     const uint32_t w = threadIdx.x >> 6;
     const uint32_t sh = 8 * (lane & 3);
 #pragma unroll
     for (int j = 0; j < U; ++j) {
-        const uint64_t ch = chunk_of<U, BLOCK>(blockIdx.x, w, j, xs);
+        const uint64_t ch = chunk_of<U, BLOCK>(b, w, j, xs);
         if (ch >= n_chunks) continue;
         const uint32_t word = c[ch * kWordsPerChunk + (lane >> 2)];
         st4<true, NT>(out + ch * kChunk + lane * 4, deq_byte((word >> sh) & 0xFFu, t));
@@ -1282,9 +1310,10 @@ struct Knobs {
     int xcd_shift;        // quantize/copy: chunks interleaved over 2^xcd_shift workgroups
     int xcd_shift_decode; // the same for dequantize (write-dominated: contiguous wins)
     int xcd_shift_acc;    // the same for the sum over payloads (tiles of 1024 elements over all 8 XCDs)
+    int decode_prefetch;  // flat decode: 0 = prefetch the code words when they cannot all be in the memory-side cache, 1 = always, 2 = never
 };
-constexpr int kKnobCount = 6;
-std::atomic<int> g_knobs[kKnobCount] = {{1}, {256}, {1}, {2}, {0}, {3}};
+constexpr int kKnobCount = 7;
+std::atomic<int> g_knobs[kKnobCount] = {{1}, {256}, {1}, {2}, {0}, {3}, {0}};
 
 thread_local Knobs tk;  // the calling thread's snapshot, taken on entry to an entry point
 
@@ -1296,6 +1325,7 @@ inline void snapshot_knobs()
     tk.xcd_shift = g_knobs[NKLQ_TUNE_XCD_INTERLEAVE_LOG2].load(std::memory_order_relaxed);
     tk.xcd_shift_decode = g_knobs[NKLQ_TUNE_XCD_INTERLEAVE_LOG2_DECODE].load(std::memory_order_relaxed);
     tk.xcd_shift_acc = g_knobs[NKLQ_TUNE_XCD_INTERLEAVE_LOG2_ACCUMULATE].load(std::memory_order_relaxed);
+    tk.decode_prefetch = g_knobs[NKLQ_TUNE_DECODE_PREFETCH].load(std::memory_order_relaxed);
 }
 
 // ---- kernel launch with the launch's own status
@@ -1437,17 +1467,33 @@ int launch_quant_flat(const float* g, const float* rin, float* rout, uint32_t* c
     return launch_status();
 }
 
+constexpr uint32_t kPrefetchLead = 16;                     // blocks of kPrefetchBlock workgroups (16 MiB of output) ahead
+constexpr uint64_t kPrefetchFromElements = 1ull << 30;     // 256 MiB of code words
+
 template <int U, int BLOCK>
 int launch_deq_flat(float* out, const uint32_t* c, uint64_t n, float t, hipStream_t s)
 {
-    const FlatGrid fg = flat_grid(n, U, BLOCK, tk.xcd_shift_decode);
+    FlatGrid fg = flat_grid(n, U, BLOCK, tk.xcd_shift_decode);
     if (fg.blocks == 0) return NKLQ_ERANGE;
+    // Prefetch workgroups (see the kernel) when the code words cannot all be in the 256 MB memory-side cache
+    // (from 2^30 elements: 1.0e9 elements still decode at 0.94 of the HBM peak without, 1.1e9 at 0.77, 1.4e9 at
+    // 0.61), or when the caller says they are not there; never for vectors of a few blocks
+    uint32_t pf_lead = 0;
+    const uint64_t work = fg.blocks - fg.has_tail;
+    const bool wanted = tk.decode_prefetch == 1 || (tk.decode_prefetch == 0 && n >= kPrefetchFromElements);
+    if (wanted && fg.xs == 0 && work >= 2 * kPrefetchLead * kPrefetchBlock) {
+        const uint64_t with = (work + kPrefetchBlock - 1) / kPrefetchBlock * (kPrefetchBlock + 8) + fg.has_tail;
+        if (with <= 0x7FFFFFFFull) {
+            fg.blocks = (uint32_t)with;
+            pf_lead = kPrefetchLead;
+        }
+    }
     if (tk.nontemporal)
         launch_kernel((deq_flat_kernel<U, BLOCK, true>), dim3(fg.blocks), dim3(BLOCK), 0, s, out, c, n,
-                      fg.n_chunks, fg.has_tail, fg.xs, t);
+                      fg.n_chunks, fg.has_tail, fg.xs, t, pf_lead);
     else
         launch_kernel((deq_flat_kernel<U, BLOCK, NKLQ_NT(false)>), dim3(fg.blocks), dim3(BLOCK), 0, s, out, c, n,
-                      fg.n_chunks, fg.has_tail, fg.xs, t);
+                      fg.n_chunks, fg.has_tail, fg.xs, t, pf_lead);
     return launch_status();
 }
 
@@ -1743,6 +1789,9 @@ int nklq_tune(int which, int value)
             if (value != 1) return NKLQ_ERANGE;
             break;
 #endif
+        case NKLQ_TUNE_DECODE_PREFETCH:
+            if (value > 2) return NKLQ_ERANGE;
+            break;
         default:
             if (value > 6) return NKLQ_ERANGE;
             break;

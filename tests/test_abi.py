@@ -145,11 +145,13 @@ def _round_trip(cases):
         _lib.tune(which, before)
     with pytest.raises(ValueError):
         _lib.tune(9, 1)
+    with pytest.raises(ValueError):
+        _lib.tune(_lib.N_TUNE, 1)
 
 
 def test_tune_knobs_round_trip():
     """The product library has one workgroup shape: its first three knobs take their default only."""
-    interleave = ((3, (0, 1, 2, 3, 4, 5, 6), (7,)), (4, (0, 3, 6), (7,)), (5, (0, 3, 6), (7,)))
+    interleave = ((3, (0, 1, 2, 3, 4, 5, 6), (7,)), (4, (0, 3, 6), (7,)), (5, (0, 3, 6), (7,)), (6, (0, 1, 2), (3,)))
     _round_trip(((0, (1,), (2, 3, 4)), (1, (256,), (64, 96, 1024)), (2, (1,), (0,))) + interleave)
     with _lib.use_tuning_library():
         _round_trip(((0, (1, 2, 4), (3,)), (1, (64, 128, 256, 512, 1024), (96,)), (2, (0, 1), ())) + interleave)

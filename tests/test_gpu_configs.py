@@ -210,6 +210,27 @@ def test_large_matrices_every_kernel_regime_against_the_oracle(n, k):
     assert_bits_equal(R.cpu().numpy(), oracle.c.dequantize(want_c, n, thrd), f"{n}x{k} decode")
 
 
+def test_flat_decode_of_more_code_words_than_the_memory_side_cache_holds():
+    """From 2^30 elements the flat decode adds prefetch workgroups by itself (the code words then
+    exceed the 256 MB cache).  4.3 GB of output: windows of it are compared with the oracle, at the
+    start (no prefetch has run yet), across block boundaries, around 2^32 bytes and at the end."""
+    n = (1 << 30) + 4099
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(30)
+    dc = torch.randint(-2 ** 31, 2 ** 31 - 1, ((n + 15) // 16,), dtype=torch.int32, device="cuda", generator=gen)
+    out = torch.full((n,), 9.0, device="cuda")
+    q.cu_fn_matrix_dequantize_e(out, dc, None, 2e-3)
+    block = 256 * 1024                     # elements of one block of 256 workgroups
+    for lo in (0, 15 * block, 16 * block - 4096, 1000 * block - 1024, (1 << 30) - (1 << 20), n - (1 << 20) - 3):
+        lo -= lo % 16
+        hi = min(n, lo + (1 << 21))
+        words = dc[lo // 16:(hi + 15) // 16].cpu().numpy().view(np.uint32)
+        assert_bits_equal(out[lo:hi].cpu().numpy(), oracle.c.dequantize(words, hi - lo, 2e-3), f"window at {lo}")
+    # and nothing but {+t, -t, +0} anywhere
+    t = torch.tensor(2e-3, dtype=torch.float32, device="cuda")
+    assert bool(((out == t) | (out == -t) | (out == 0)).all())
+
+
 @pytest.mark.parametrize("n,k", [(46_349, 46_341), (268_435_461, 9)])
 def test_matrix_forms_beyond_2_31_elements(n, k):
     """Matrices of more than 2^31 elements (8.6 and 9.7 GB per array) through the row kernels and

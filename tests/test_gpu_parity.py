@@ -475,6 +475,39 @@ def _turn_the_knobs_while_another_thread_launches():
 
 
 
+@pytest.mark.parametrize("n", [8_388_608, 8_388_608 + 5, 20_000_003, (256 + 8) * 1024 * 40 + 777])
+def test_flat_decode_with_prefetching_workgroups(n):
+    """The flat decode with its prefetch workgroups switched on (the library does that by itself only
+    from 2^30 elements): 8 extra workgroups behind every 256, which only read code words ahead; the
+    256 in front must still write exactly their pieces.  Product geometry and two others."""
+    rng = np.random.default_rng(n % 1000)
+    words = rng.integers(0, 2 ** 32, size=(n + 15) // 16, dtype=np.uint64).astype(np.uint32)
+    want = oracle.c.dequantize(words, n, 3e-3)
+    dc = dev(words)
+    old = _lib.tune(_lib.TUNE_DECODE_PREFETCH)
+    try:
+        for mode in (1, 2, 0):
+            _lib.tune(_lib.TUNE_DECODE_PREFETCH, mode)
+            out = torch.full((n,), 9.0, device="cuda")
+            q.cu_fn_matrix_dequantize_e(out, dc, None, 3e-3)
+            assert_bits_equal(out.cpu().numpy(), want, f"n={n} prefetch knob {mode}")
+    finally:
+        _lib.tune(_lib.TUNE_DECODE_PREFETCH, old)
+    with _lib.use_tuning_library():
+        old = [_lib.tune(i) for i in range(_lib.N_TUNE)]
+        try:
+            _lib.tune(_lib.TUNE_DECODE_PREFETCH, 1)
+            for u, wg in ((2, 128), (1, 512)):
+                _lib.tune(_lib.TUNE_CHUNKS_PER_WAVE, u)
+                _lib.tune(_lib.TUNE_WORKGROUP_SIZE, wg)
+                out = torch.full((n,), 9.0, device="cuda")
+                q.cu_fn_matrix_dequantize_e(out, dc, None, 3e-3)
+                assert_bits_equal(out.cpu().numpy(), want, f"n={n} prefetch, {u} chunks per wave, workgroup {wg}")
+        finally:
+            for i, v in enumerate(old):
+                _lib.tune(i, v)
+
+
 def test_empty_inputs_are_no_ops():
     e = torch.empty(0, device="cuda")
     w = torch.empty(0, dtype=torch.int32, device="cuda")
