@@ -157,9 +157,13 @@ class GradCompressor:
         contiguous temporary) pairs for tensors that are not contiguous (their temporary is what the
         kernels see).
 
-        Gradients normally keep their storage from step to step, so the tables are cached on the
+        Gradients normally keep their storage from step to step (also when `.grad` is a new tensor
+        object every step: the allocator hands out the same blocks), so the tables are cached on the
         tuple of their addresses: a steady-state call costs one pass that reads the addresses and
-        nothing else (no ctypes arrays are rebuilt, no tensor is examined again)."""
+        nothing else (no ctypes arrays are rebuilt, no tensor is examined again).  Sizes and types
+        are looked at when an address changes, not on a hit: they belong to the parameter, not to
+        the step, and a tensor of another size at the very address its predecessor had is taken
+        for the predecessor."""
         if len(tensors) != len(self.layout):
             raise ValueError(f"expected {len(self.layout)} {what}s, got {len(tensors)}")
         try:
