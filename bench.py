@@ -780,7 +780,7 @@ def main():
                     sizes += [4 * planes * inpl, 4 * planes, 4 * planes]
                 inpl = 4 * planes
         sizes += [1000 * 2048, 1000]
-        gcomp = ptcomp.GradCompressor(sizes, K_PAYLOADS, thrd=THRD)
+        gcomp = ptcomp.GradCompressor(sizes, K_PAYLOADS, thrd=THRD, rank=0)
         gl, pos = [], 0
         for sz in sizes:
             gl.append(g[pos:pos + sz])

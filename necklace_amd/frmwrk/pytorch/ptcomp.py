@@ -113,19 +113,29 @@ class GradCompressor:
     """Flat buffers + the compress / decompress steps for one model replica."""
 
     def __init__(self, params, kn, thrd=DEFAULT_COMP_THRESHOLD, size_threshold=DEFAULT_SIZE_THRESHOLD,
-                 device="cuda", rank=0):
+                 device="cuda", rank=None):
+        """`rank`: this worker's index among the kn.  Known, this rank's payload is written straight
+        into its own slot of the receive buffer (the all-gather can then run in place).  None with
+        several workers (the reference's set-up call, necklace/trainer/tnopmx.py:140-143, does not
+        pass one): the payload gets a buffer of its own, and whatever needs to know who this worker
+        is (a reduce onto a root) raises instead of assuming worker 0."""
         if kn < 1:
             raise ValueError("kn (number of workers) must be >= 1")
-        if not 0 <= rank < kn:
+        if rank is None and kn == 1:
+            rank = 0
+        if rank is not None and not 0 <= rank < kn:
             raise ValueError("rank must be in [0, kn)")
-        self.kn, self.rank, self.thrd = int(kn), int(rank), float(thrd)
+        self.kn, self.rank, self.thrd = int(kn), (None if rank is None else int(rank)), float(thrd)
         self.layout = GradCompLayout([_numel(p) for p in params], size_threshold)
         lay = self.layout
         self.device = torch.device(device)
         self.resi = torch.zeros(lay.total_elems, dtype=torch.float32, device=self.device)
         # slot k of `recv` holds rank k's payload; this rank's own slot doubles as `comp`
         self.recv = torch.zeros(self.kn, max(lay.total_words, 1), dtype=torch.int32, device=self.device)
-        self.comp = self.recv[self.rank, :lay.total_words]
+        if self.rank is None:
+            self.comp = torch.zeros(max(lay.total_words, 1), dtype=torch.int32, device=self.device)[:lay.total_words]
+        else:
+            self.comp = self.recv[self.rank, :lay.total_words]
         self.grd_cmps = list(lay.compressed)
         self.grd_resi, self.grd_comp, self.grd_recv = [], [], []
         for i in range(len(lay)):
@@ -307,29 +317,36 @@ def quantize_chunked(g, c, r, thrd, chunk=DEFAULT_CHUNK, stream=None, add_residu
 
 # --------------------------------------------------------------------------- functional surface
 
-def init_grads_compression(params, kn, grd_siz_thrd=DEFAULT_SIZE_THRESHOLD, device="cuda", rank=0,
+def init_grads_compression(params, kn, grd_siz_thrd=DEFAULT_SIZE_THRESHOLD, device="cuda", rank=None,
                            thrd=DEFAULT_COMP_THRESHOLD):
     """Counterpart of the call at necklace/trainer/tnopmx.py:140-143.
 
     Returns ``(grd_resi, grd_recv, grd_comp, grd_cmps)``: per-parameter residuals,
-    ``[kn, words]`` receive slots, local packed codes (views of this rank's receive slot), and
-    which parameters are compressed.  The views keep the flat buffers alive; use
+    ``[kn, words]`` receive slots, local packed codes (views of this rank's receive slot when `rank`
+    is given, of a buffer of their own otherwise), and which parameters are compressed.  The views keep the flat buffers alive; use
     `init_grad_comp_cfg` to also get the `GradCompressor` that owns them.
     """
     gc = GradCompressor(params, kn, thrd=thrd, size_threshold=grd_siz_thrd, device=device, rank=rank)
     return gc.grd_resi, gc.grd_recv, gc.grd_comp, gc.grd_cmps
 
 
-def init_grad_comp_cfg(params, kn, grad_comp_cfg=None, device="cuda", rank=0):
+def init_grad_comp_cfg(params, kn, grad_comp_cfg=None, device="cuda", rank=None):
     """Fill a ``grad_comp_cfg`` dict the way TrainerOPMxnet.init_grads_comp does
     (necklace/trainer/tnopmx.py:135-151): keys grd_resi, grd_recv, grd_comp, grd_cmps,
-    grad_size_threshold, grad_comp_threshold; plus 'compressor', the object that owns the buffers."""
+    grad_size_threshold, grad_comp_threshold; plus 'compressor', the object that owns the buffers.
+    `rank` (or ``grad_comp_cfg['rank']``): see GradCompressor; it is recorded in the dict."""
     cfg = dict(grad_comp_cfg or {})
+    if "rank" in cfg:
+        if rank is not None and int(rank) != int(cfg["rank"]):
+            raise ValueError(f"rank = {rank} but grad_comp_cfg['rank'] = {cfg['rank']}")
+        rank = int(cfg["rank"])
     siz = cfg.get("grad_size_threshold", DEFAULT_SIZE_THRESHOLD)
     thr = cfg.get("grad_comp_threshold", DEFAULT_COMP_THRESHOLD)
     gc = GradCompressor(params, kn, thrd=thr, size_threshold=siz, device=device, rank=rank)
     cfg.update(grd_resi=gc.grd_resi, grd_recv=gc.grd_recv, grd_comp=gc.grd_comp, grd_cmps=gc.grd_cmps,
                grad_size_threshold=siz, grad_comp_threshold=thr, compressor=gc)
+    if gc.rank is not None:
+        cfg["rank"] = gc.rank
     return cfg
 
 
@@ -376,7 +393,7 @@ def grads_do_compressed_exchange(grads, kn, grad_comp_cfg, exchange=None, averag
 
 # --------------------------------------------------------------------------- flat gradient buffer
 
-def init_flat_grad_comp_cfg(total_size, kn, grad_comp_cfg=None, device="cuda", rank=0):
+def init_flat_grad_comp_cfg(total_size, kn, grad_comp_cfg=None, device="cuda", rank=None):
     """`grad_comp_cfg` for ONE flat gradient buffer of `total_size` floats — the `grd_fltn_gpu` of
     PtCudaFltnMemManager (necklace/frmwrk/pytorch/tsmem.py:157-180), which the flat ZeRO trainer
     reduces as a whole (necklace/trainer/zroppf.py:957-965).  Residual, payload and receive slots
@@ -551,6 +568,17 @@ def _rank_of(nc, cfg, kn):
     return 0
 
 
+def _decodes(gc, root):
+    """Whether this worker decodes the sum: every worker of an all-reduce (root None), the root of a
+    reduce.  A compressor that was set up without a rank cannot tell and says so."""
+    if root is None:
+        return True
+    if gc.rank is None:
+        raise ValueError("a reduce onto a root needs this worker's rank: set grad_comp_cfg['rank'] "
+                         "(or pass rank= where the buffers are set up)")
+    return gc.rank == root
+
+
 def _check_fp32(grads):
     """The compressed path packs fp32 gradients.  The reference buckets per tensor type
     (_take_tensors, necklace/frmwrk/pytorch/ptprms.py:258) and all-reduces every type; here any other
@@ -592,8 +620,9 @@ def _cfg_for_params(params, kn, cfg, nc=None):
         if old_gc is not None and "_signature" not in cfg and old_gc.kn == kn \
                 and old_gc.layout.numels == numels and old_gc.layout.size_threshold == siz:
             gc = old_gc  # laid out beforehand for exactly these parameters
-            if "rank" in cfg and int(cfg["rank"]) != gc.rank:
-                raise ValueError(f"grad_comp_cfg['rank'] = {cfg['rank']}, its buffers were laid out for rank {gc.rank}")
+            known = int(cfg["rank"]) if "rank" in cfg else getattr(nc, "rank", None)
+            if known is not None and not callable(known) and gc.rank is not None and int(known) != gc.rank:
+                raise ValueError(f"this worker's rank is {known}, the buffers were laid out for rank {gc.rank}")
         else:
             dev = params[0].device if params else torch.device("cuda")
             built = init_grad_comp_cfg(params, kn, cfg, device=dev, rank=_rank_of(nc, cfg, kn))
@@ -636,7 +665,7 @@ def _reduce_params_form(nc, kn, root, params, cfg):
     average = root is None  # the reference's reduce leaves `/ kn` commented out (ptprms.py:385)
     gc.compress(grads)
     _run_exchange(_exchange_of(nc), gc, kn, None)
-    if root is None or gc.rank == root:
+    if _decodes(gc, root):
         gc.decompress_sum(grads, average=average)
     small = [g for g, c in zip(grads, gc.grd_cmps) if g is not None and not c]
     _reduce_small(small, kn, _small_fn(nc, cfg, root), average)
@@ -695,7 +724,7 @@ def _reduce_buckets_form(nc, kn, root, params, cfg):
         torch.cat([g.reshape(-1) for g in bucket], out=flat)
     gc.compress(flats)
     _run_exchange(_exchange_of(nc), gc, kn, None)
-    if root is None or gc.rank == root:
+    if _decodes(gc, root):
         gc.decompress_sum(flats, average=root is None)
         for flat, bucket in zip(flats, buckets):  # unflatten and copy back, ptprms.py:296-299
             pos = 0
@@ -795,4 +824,4 @@ def opt_grads_fltn_do_nccl_reduce(nc, kn, root, d_arr_send, sz, grad_comp_cfg=No
         gc = grad_comp_cfg["compressor"]
         _apply_pending_state(grad_comp_cfg, gc)
     opt_grads_fltn_do_compressed_reduce(kn, d_arr_send, sz, grad_comp_cfg, exchange=_exchange_of(nc),
-                                        average=False, decode=gc.rank == root)
+                                        average=False, decode=_decodes(gc, root))

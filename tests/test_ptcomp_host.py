@@ -194,9 +194,38 @@ def test_rank_is_required_with_several_workers():
         ptcomp._cfg_for_params(params, 2, {})
     with pytest.raises(ValueError):
         ptcomp.opt_grads_fltn_do_nccl_reduce(None, 2, 0, torch.zeros(64), 64, grad_comp_cfg={})
-    cfg = ptcomp.init_grad_comp_cfg(params, 2, {"rank": 1}, device="cpu", rank=0)
-    with pytest.raises(ValueError):                      # the dict says 1, the buffers were laid out for 0
-        ptcomp._cfg_for_params(params, 2, cfg)
+    with pytest.raises(ValueError):                      # the dict says 1, the argument 0
+        ptcomp.init_grad_comp_cfg(params, 2, {"rank": 1}, device="cpu", rank=0)
+    cfg = ptcomp.init_grad_comp_cfg(params, 2, {}, device="cpu", rank=0)
+    assert cfg["rank"] == 0
+    rankless = {k: v for k, v in cfg.items() if k != "rank"}
+
+    class Other:
+        rank = 1
+    with pytest.raises(ValueError):                      # the communicator says 1, the buffers were laid out for 0
+        ptcomp._cfg_for_params(params, 2, rankless, Other())
+
+
+def test_buffers_set_up_without_a_rank_assume_none():
+    """The reference's set-up call passes no rank (necklace/trainer/tnopmx.py:140-143).  The payload then
+    has a buffer of its own instead of a slot of the receive buffer, and a reduce onto a root, which has
+    to know who this worker is, raises; nothing ever assumes worker 0."""
+    params = _params(3000, 5000)
+    resi, recv, comp, cmps = ptcomp.init_grads_compression(params, 4, device="cpu")
+    gc_rankless = ptcomp.GradCompressor([3000, 5000], kn=4, device="cpu")
+    assert gc_rankless.rank is None
+    lo, hi = gc_rankless.recv.data_ptr(), gc_rankless.recv.data_ptr() + 4 * gc_rankless.recv.numel()
+    assert not lo <= gc_rankless.comp.data_ptr() < hi          # not a slot of the receive buffer
+    assert all(not lo <= c.data_ptr() < hi for c in gc_rankless.grd_comp if c is not None)
+    gc1 = ptcomp.GradCompressor([3000], kn=1, device="cpu")
+    assert gc1.rank == 0 and gc1.comp.data_ptr() == gc1.recv.data_ptr()
+    gc2 = ptcomp.GradCompressor([3000], kn=4, device="cpu", rank=2)
+    assert gc2.comp.data_ptr() == gc2.recv[2].data_ptr()
+    with pytest.raises(ValueError, match="rank"):
+        ptcomp._decodes(gc_rankless, 0)
+    assert ptcomp._decodes(gc_rankless, None) and ptcomp._decodes(gc2, 2) and not ptcomp._decodes(gc2, 1)
+    cfg = ptcomp.init_grad_comp_cfg(params, 4, {}, device="cpu")
+    assert "rank" not in cfg and cfg["compressor"].rank is None
 
 
 def test_gradients_that_are_not_float32_are_refused_up_front():
