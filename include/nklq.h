@@ -171,12 +171,13 @@ int nklq_version(void);
                                             workgroups (which run on different XCDs): 0..6 */
 #define NKLQ_TUNE_XCD_INTERLEAVE_LOG2_DECODE 4  /* the same for dequantize */
 #define NKLQ_TUNE_XCD_INTERLEAVE_LOG2_ACCUMULATE 5  /* the same for the tiles (1024 elements) of the sum over payloads */
-#define NKLQ_TUNE_DECODE_PREFETCH 6      /* flat dequantize: extra workgroups read the code words ahead of the
-                                            decoding ones.  Pays when the words come from HBM (0.6 -> 0.88 of
-                                            the HBM peak), costs 6 % when they are in the 256 MB memory-side
-                                            cache anyway (just written or read).  0: only for vectors whose
-                                            words exceed that cache (2^30 elements and more); 1: always;
-                                            2: never */
+#define NKLQ_TUNE_DECODE_PREFETCH 6      /* dequantize with code words that are not in the 256 MB memory-side
+                                            cache.  Flat: extra workgroups read the words ahead of the decoding
+                                            ones; matrix: ranges of bands, each behind a pass over its words.
+                                            Pays when the words come from HBM (0.6 -> 0.85-0.9 of the HBM
+                                            peak), costs 6 % when they are in that cache anyway (just written
+                                            or read).  0: only for inputs whose words exceed the cache (2^30
+                                            elements and more); 1: always; 2: never */
 int nklq_tune(int which, int value);
 
 #ifdef __cplusplus

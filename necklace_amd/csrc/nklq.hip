@@ -1734,6 +1734,21 @@ bool mul_ok(uint64_t a, uint64_t b, uint64_t* out)
     return true;
 }
 
+// One word of every 128-byte line of `words` code words is read (and dropped): the lines are then in
+// the memory-side cache for the decode that follows on the same stream.
+__global__ __launch_bounds__(256) void touch_words_kernel(const uint32_t* __restrict__ c, uint64_t words)
+{
+    const uint64_t wi = ((uint64_t)blockIdx.x * 256 + threadIdx.x) * 32;
+    if (wi < words) {
+        const uint32_t bits = c[wi];
+        asm volatile("" : : "v"(bits));
+    }
+}
+constexpr uint64_t kTouchRangeWords = 1ull << 24;      // 64 MiB of code words per range: a quarter of the memory-side cache
+constexpr uint64_t kTouchFromElements = 1ull << 24;    // smaller matrices are decoded as they are
+
+int decode_matrix(float* out, const uint32_t* c, uint64_t n_rows, uint64_t n_cols, float thrd, hipStream_t s);
+
 }  // namespace
 
 // ---------------------------------------------------------------- C-ABI
@@ -1946,6 +1961,39 @@ int nklq_dequantize_f32(float* out, const uint32_t* c, uint64_t n_rows, uint64_t
     if (n_cols == 1) {
         return dispatch_deq_flat(out, c, total, thrd, s);
     }
+    // The matrix decodes are as sensitive to where their code words come from as the flat one (see
+    // deq_flat_kernel): 16384 x 16383 runs at 0.92 of the HBM peak with the words in the memory-side cache and
+    // at 0.58 with the words in HBM.  When they cannot all be in that cache, or the caller says they are not, the
+    // matrix is decoded in ranges of bands of at most 64 MiB of words, each right after a pass that reads one
+    // word of every line of the range's words (touch_words_kernel): that pass costs the words' share of the bytes.
+    const bool touch = tk.decode_prefetch == 1 || (tk.decode_prefetch == 0 && total >= kPrefetchFromElements);
+    if (touch && total >= kTouchFromElements) {
+        uint64_t bands = kTouchRangeWords / n_cols / 8 * 8;   // whole groups of 8 bands (the tile maps deal bands in eights)
+        if (bands < 8) bands = 8;
+        const uint64_t rows = bands * 16;
+        for (uint64_t r0 = 0; r0 < n_rows; r0 += rows) {
+            const uint64_t nr = n_rows - r0 < rows ? n_rows - r0 : rows;
+            const uint32_t* cr = c + (r0 / 16) * n_cols;
+            const uint64_t words = nklq_packed_words(nr, n_cols);
+            const uint64_t lines = (words + 31) / 32;
+            const uint64_t tb = (lines + 255) / 256;
+            if (tb > 0x7FFFFFFFull) return NKLQ_ERANGE;
+            launch_kernel(touch_words_kernel, dim3((uint32_t)tb), dim3(256), 0, s, cr, words);
+            if (launch_status() != NKLQ_OK) return launch_status();
+            const int st = decode_matrix(out + r0 * n_cols, cr, nr, n_cols, thrd, s);
+            if (st != NKLQ_OK) return st;
+        }
+        return NKLQ_OK;
+    }
+    return decode_matrix(out, c, n_rows, n_cols, thrd, s);
+}
+
+}  // extern "C"
+
+namespace {
+
+int decode_matrix(float* out, const uint32_t* c, uint64_t n_rows, uint64_t n_cols, float thrd, hipStream_t s)
+{
     const uint64_t m = n_rows / 16 + (n_rows % 16 ? 1 : 0);
     if (16 * n_cols <= kBandsDecodeWholeMax) {
         // short bands: the fewest whole bands that give every lane of the workgroup a quad
@@ -2007,6 +2055,10 @@ int nklq_dequantize_f32(float* out, const uint32_t* c, uint64_t n_rows, uint64_t
                       (uint32_t)pieces, inv_pieces, inv_k, thrd, pinned);
     return launch_status();
 }
+
+}  // namespace
+
+extern "C" {
 
 int nklq_dequant_accumulate_f32(float* acc, const uint32_t* const* payloads, int k_payloads,
                                 uint64_t n, float thrd, int accumulate, void* stream)

@@ -231,6 +231,33 @@ def test_flat_decode_of_more_code_words_than_the_memory_side_cache_holds():
     assert bool(((out == t) | (out == -t) | (out == 0)).all())
 
 
+@pytest.mark.parametrize("n,k", [(4099, 8191), (20_011, 1023), (1_000_003, 17), (40_000, 8191), (300, 100_003)])
+def test_matrix_decode_in_ranges_behind_a_pass_over_the_code_words(n, k):
+    """With the prefetch knob on, a matrix of 2^24 elements or more is decoded in ranges of bands
+    (at most 64 MiB of code words each; 40,000 x 8191 takes two, 300 x 100,003 three), each behind a
+    pass that reads the range's words.  Same bits as the decode in one piece, and as the oracle
+    on windows that include the seams."""
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(n + k)
+    C = torch.randint(-2 ** 31, 2 ** 31 - 1, ((n + 15) // 16, k), dtype=torch.int32, device="cuda", generator=gen)
+    one, ranged = torch.full((n, k), 9.0, device="cuda"), torch.full((n, k), 9.0, device="cuda")
+    old = _lib.tune(_lib.TUNE_DECODE_PREFETCH)
+    try:
+        _lib.tune(_lib.TUNE_DECODE_PREFETCH, 2)
+        q.cu_fn_matrix_dequantize_e(one, C, None, 2e-3)
+        _lib.tune(_lib.TUNE_DECODE_PREFETCH, 1)
+        q.cu_fn_matrix_dequantize_e(ranged, C, None, 2e-3)
+    finally:
+        _lib.tune(_lib.TUNE_DECODE_PREFETCH, old)
+    assert torch.equal(one.view(torch.int32), ranged.view(torch.int32))
+    bands = max(8, (1 << 24) // k // 8 * 8)
+    for r0 in (0, 16 * bands - 16, n - min(n, 48)):
+        r0 = max(0, min(r0, n - 1)) // 16 * 16
+        r1 = min(n, r0 + 48)
+        words = C[r0 // 16:(r1 + 15) // 16].cpu().numpy().view(np.uint32)
+        assert_bits_equal(ranged[r0:r1].cpu().numpy(), oracle.c.dequantize(words, r1 - r0, 2e-3), f"rows {r0}..{r1}")
+
+
 @pytest.mark.parametrize("n,k", [(46_349, 46_341), (268_435_461, 9)])
 def test_matrix_forms_beyond_2_31_elements(n, k):
     """Matrices of more than 2^31 elements (8.6 and 9.7 GB per array) through the row kernels and
